@@ -1,0 +1,189 @@
+/*
+ * C ABI of the MI355X (gfx950) stochastic-rounding AdamW library.
+ *
+ * Plain C types only: pointers, sizes, enums-as-int.  Every entry point
+ * returns 0 on success or a negative RT_E* code; rt_last_error() then holds a
+ * message (with the hipError_t text where one was involved).  No exception or
+ * torch type crosses this boundary.  The caller owns every tensor pointer it
+ * passes in; the library owns only its handle's private workspace.
+ *
+ * The reference is pure Python on torch and has no FFI of its own; each entry
+ * point cites the reference code whose work it takes over.
+ */
+#ifndef RAMTORCH_SR_ADAMW_H
+#define RAMTORCH_SR_ADAMW_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RT_ABI_VERSION 1
+
+/* error codes */
+#define RT_OK 0
+#define RT_EINVAL (-1)   /* bad argument (null pointer, unknown dtype, bad offset ...) */
+#define RT_EHIP (-2)     /* a HIP runtime call failed; see rt_last_error() */
+#define RT_ENOMEM (-3)   /* workspace allocation failed */
+#define RT_EUNSUPPORTED (-4) /* valid request the kernels do not implement */
+
+/* element types */
+#define RT_DT_BF16 0
+#define RT_DT_F32 1
+#define RT_DT_F16 2 /* gradients only */
+
+/* where the rounding noise comes from */
+#define RT_NOISE_PHILOX 0   /* Philox4x32-10 keyed by seed; counter from (step, tensor, element) */
+#define RT_NOISE_EXPLICIT 1 /* caller-supplied int16/uint16 noise per element and array */
+
+/* rt_tensor_desc.host_mask bits: array lives in host memory (streamed entry point only) */
+#define RT_HOST_P 1u
+#define RT_HOST_G 2u
+#define RT_HOST_M 4u
+#define RT_HOST_V 8u
+
+/*
+ * Per-(param group, step) constants: the Python doubles of
+ * ramtorch/stochastic_optimizers/adamw.py:173-188, each already rounded to
+ * float32 exactly where an ATen call of adamw.py:190-200 would round it.
+ */
+typedef struct rt_scalars {
+    float beta1;          /* float32(beta1)                      adamw.py:190 */
+    float one_m_beta1;    /* float32(1 - beta1)                  adamw.py:190 */
+    float beta2;          /* float32(beta2)                      adamw.py:191 */
+    float one_m_beta2;    /* float32(1 - beta2)                  adamw.py:191 */
+    float inv_bcs;        /* 1.0f / float32(sqrt(1 - beta2^t))   adamw.py:187,193 */
+    float eps;            /* float32(eps)                        adamw.py:194 */
+    float decay;          /* float32(1 - (lr/bc) * wd)           adamw.py:188,198 */
+    float neg_step_size;  /* float32(-(lr/bc))                   adamw.py:188,200 */
+    float inv_loss_scale; /* grads are multiplied by this first; 1.0f = off (not in the reference) */
+    float centralization; /* float32(centralization)             adamw.py:176-184; 0 = off */
+    int32_t apply_decay;  /* weight_decay != 0                   adamw.py:197 */
+    int32_t reserved;
+} rt_scalars;
+
+/*
+ * One parameter tensor (or one contiguous piece of one).  p/m/v are updated in
+ * place.  For rt_step_multi every pointer is a device address; for
+ * rt_step_streamed the arrays named in host_mask are host addresses.
+ */
+typedef struct rt_tensor_desc {
+    void* p;               /* parameter            adamw.py:168-170, 204-214 */
+    const void* g;         /* gradient             adamw.py:117, 167 */
+    void* m;               /* state["ema"]         adamw.py:160, 215-222 */
+    void* v;               /* state["ema_squared"] adamw.py:163, 215-222 */
+    const void* noise_p;   /* RT_NOISE_EXPLICIT: numel 16-bit noises per bf16 array, else NULL */
+    const void* noise_m;
+    const void* noise_v;
+    float* dbg_p;          /* optional device fp32[numel]: values before rounding (tests) */
+    float* dbg_m;
+    float* dbg_v;
+    const float* row_mean; /* centralization != 0: device fp32[numel/row_len] row means of g */
+    uint64_t numel;
+    uint64_t elem_offset;  /* index of element 0 inside the logical tensor; multiple of 8 */
+    uint64_t row_len;      /* elements per row (dim 0 slice) when row_mean != NULL */
+    uint32_t tensor_id;    /* < 2^30; part of the Philox counter */
+    uint32_t step;         /* state["step"] after the increment (adamw.py:177), mod 2^32 */
+    uint32_t scalars_idx;  /* index into the rt_scalars array */
+    uint8_t p_dtype;       /* RT_DT_BF16 (stochastic rounding) or RT_DT_F32 (plain store) */
+    uint8_t g_dtype;       /* RT_DT_BF16, RT_DT_F32 or RT_DT_F16 */
+    uint8_t m_dtype;       /* RT_DT_BF16 or RT_DT_F32 */
+    uint8_t v_dtype;       /* RT_DT_BF16 or RT_DT_F32 */
+    uint32_t host_mask;    /* RT_HOST_* bits; must be 0 for rt_step_multi */
+    uint32_t reserved;
+} rt_tensor_desc;
+
+typedef struct rt_handle rt_handle;
+
+/* ABI version of the loaded library (RT_ABI_VERSION it was built with). */
+int rt_version(void);
+
+/* Message of the calling thread's most recent failure ("" if none). */
+const char* rt_last_error(void);
+
+/*
+ * Workspace for one device: table staging, reduction scratch and, on first
+ * streamed use, three streams plus double-buffered device staging.
+ * Replaces nothing in the reference (it allocates temporaries per tensor,
+ * adamw.py:160-170); a handle is not re-entrant, distinct handles are independent.
+ */
+int rt_create(int device, rt_handle** out);
+int rt_destroy(rt_handle* h);
+
+/*
+ * The fused step over n device-resident tensors in one launch per dtype
+ * combination: replaces the per-tensor loop body of AdamW.step,
+ * adamw.py:160-222 (upcast, EMA updates, denominator, decoupled decay,
+ * addcdiv, three copy_stochastic_ write-backs) and the syncs of :227-232.
+ * Enqueues on `stream` (a hipStream_t; NULL = default stream) and returns
+ * without synchronising.
+ *   d_clip_coef: optional device float; when non-NULL grads are multiplied by
+ *                *d_clip_coef after unscaling (global-norm clip, not in the reference)
+ *   d_skip:      optional device uint32; when non-NULL and *d_skip != 0 the
+ *                launch leaves every tensor untouched (non-finite grad norm)
+ */
+int rt_step_multi(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
+                  uint32_t n_scalars, uint64_t seed, int noise_mode, const float* d_clip_coef,
+                  const uint32_t* d_skip, void* stream);
+
+/*
+ * Same update for tensors whose p/m/v (and optionally g) live in pinned host
+ * memory: the CPU-resident flow of adamw.py:152-170 (H2D of ema, ema_squared,
+ * grad, p) and :204-222 (D2H write-back), restructured as chunks of
+ * `chunk_elems` elements moved H2D / updated / moved D2H on three streams with
+ * two staging buffers per array.  Waits for work already queued on `stream`
+ * (grads ready) and returns after the last D2H has completed, so host memory
+ * is final on return (the post-condition of the sync at adamw.py:232).
+ * Results are bit-identical to rt_step_multi on the same data.
+ */
+int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
+                     uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems,
+                     void* stream);
+
+/*
+ * Global gradient norm over n device tensors (uses g, g_dtype, numel of each
+ * desc), for the optional clip / skip check; not in the reference.  Writes to
+ * d_out (device, 16-byte aligned):
+ *   float  d_out[0] = total L2 norm of g * inv_loss_scale
+ *   float  d_out[1] = min(1, max_norm / (total + 1e-6))   (torch clip_grad_norm_ semantics)
+ *   uint32 d_out[2] = 1 if the norm is not finite, else 0
+ * Two deterministic passes (per-workgroup partials, then one reducing
+ * workgroup); no atomics, so the result is reproducible run to run.
+ */
+int rt_grad_norm(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, float inv_loss_scale,
+                 float max_norm, void* d_out, void* stream);
+
+/*
+ * Row means of g over all dims but the first, for gradient centralization
+ * (adamw.py:179-184): d_row_mean[r] = mean(g[r, ...]) in fp32.
+ */
+int rt_row_means(rt_handle* h, const void* g, int g_dtype, uint64_t rows, uint64_t row_len,
+                 float inv_loss_scale, float* d_row_mean, void* stream);
+
+/*
+ * copy_stochastic_(target, source, seed) of adamw.py:6-30: fp32 device source
+ * -> bf16 device target.  noise == NULL: Philox keyed by seed; else explicit
+ * 16-bit noise per element.
+ */
+int rt_sr_copy(void* target_bf16, const float* source, uint64_t numel, const void* noise,
+               uint64_t seed, void* stream);
+
+/*
+ * Timing of the most recent rt_step_multi on this handle, measured with HIP
+ * events recorded on the launch stream around the update kernels only.
+ * Blocks until that work has finished.  Enabled by rt_set_timing(h, 1).
+ */
+int rt_set_timing(rt_handle* h, int enabled);
+int rt_last_kernel_ms(rt_handle* h, float* ms);
+
+/*
+ * Streamed-path statistics of the most recent rt_step_streamed:
+ * out[0] = bytes H2D, out[1] = bytes D2H, out[2] = wall seconds of the call.
+ */
+int rt_streamed_stats(rt_handle* h, double out[3]);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RAMTORCH_SR_ADAMW_H */

@@ -1,0 +1,191 @@
+"""ctypes binding of the C ABI in ``include/ramtorch_sr_adamw.h``.
+
+The library is the only implementation of the step: if it is missing or does
+not load, every entry point raises -- there is no fallback path.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "_lib", "libramtorch_sr_adamw.so")
+
+ABI_VERSION = 1
+
+RT_OK = 0
+RT_EINVAL, RT_EHIP, RT_ENOMEM, RT_EUNSUPPORTED = -1, -2, -3, -4
+RT_DT_BF16, RT_DT_F32, RT_DT_F16 = 0, 1, 2
+RT_NOISE_PHILOX, RT_NOISE_EXPLICIT = 0, 1
+RT_HOST_P, RT_HOST_G, RT_HOST_M, RT_HOST_V = 1, 2, 4, 8
+
+#: every symbol the header declares
+EXPORTS = (
+    "rt_version", "rt_last_error", "rt_create", "rt_destroy", "rt_step_multi", "rt_step_streamed",
+    "rt_grad_norm", "rt_row_means", "rt_sr_copy", "rt_set_timing", "rt_last_kernel_ms", "rt_streamed_stats",
+)
+
+
+class RtScalars(ctypes.Structure):
+    _fields_ = [
+        ("beta1", ctypes.c_float),
+        ("one_m_beta1", ctypes.c_float),
+        ("beta2", ctypes.c_float),
+        ("one_m_beta2", ctypes.c_float),
+        ("inv_bcs", ctypes.c_float),
+        ("eps", ctypes.c_float),
+        ("decay", ctypes.c_float),
+        ("neg_step_size", ctypes.c_float),
+        ("inv_loss_scale", ctypes.c_float),
+        ("centralization", ctypes.c_float),
+        ("apply_decay", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+    ]
+
+
+class RtTensorDesc(ctypes.Structure):
+    _fields_ = [
+        ("p", ctypes.c_void_p),
+        ("g", ctypes.c_void_p),
+        ("m", ctypes.c_void_p),
+        ("v", ctypes.c_void_p),
+        ("noise_p", ctypes.c_void_p),
+        ("noise_m", ctypes.c_void_p),
+        ("noise_v", ctypes.c_void_p),
+        ("dbg_p", ctypes.c_void_p),
+        ("dbg_m", ctypes.c_void_p),
+        ("dbg_v", ctypes.c_void_p),
+        ("row_mean", ctypes.c_void_p),
+        ("numel", ctypes.c_uint64),
+        ("elem_offset", ctypes.c_uint64),
+        ("row_len", ctypes.c_uint64),
+        ("tensor_id", ctypes.c_uint32),
+        ("step", ctypes.c_uint32),
+        ("scalars_idx", ctypes.c_uint32),
+        ("p_dtype", ctypes.c_uint8),
+        ("g_dtype", ctypes.c_uint8),
+        ("m_dtype", ctypes.c_uint8),
+        ("v_dtype", ctypes.c_uint8),
+        ("host_mask", ctypes.c_uint32),
+        ("reserved", ctypes.c_uint32),
+    ]
+
+
+assert ctypes.sizeof(RtScalars) == 48
+assert ctypes.sizeof(RtTensorDesc) == 136
+
+
+class NativeError(RuntimeError):
+    """A C-ABI call returned a non-zero code."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"ramtorch_sr_adamw error {code}: {message}")
+        self.code = code
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    """Load the shared library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: the HIP extension has not been built. "
+            "Run `python -m ramtorch_amd.build` (needs hipcc); there is no fallback implementation.")
+    L = ctypes.CDLL(LIB_PATH)
+    vp, u32, u64, i32 = ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_int
+    descs, scal = ctypes.POINTER(RtTensorDesc), ctypes.POINTER(RtScalars)
+    L.rt_version.restype = i32
+    L.rt_version.argtypes = []
+    L.rt_last_error.restype = ctypes.c_char_p
+    L.rt_last_error.argtypes = []
+    L.rt_create.restype = i32
+    L.rt_create.argtypes = [i32, ctypes.POINTER(vp)]
+    L.rt_destroy.restype = i32
+    L.rt_destroy.argtypes = [vp]
+    L.rt_step_multi.restype = i32
+    L.rt_step_multi.argtypes = [vp, descs, u32, scal, u32, u64, i32, vp, vp, vp]
+    L.rt_step_streamed.restype = i32
+    L.rt_step_streamed.argtypes = [vp, descs, u32, scal, u32, u64, i32, u64, vp]
+    L.rt_grad_norm.restype = i32
+    L.rt_grad_norm.argtypes = [vp, descs, u32, ctypes.c_float, ctypes.c_float, vp, vp]
+    L.rt_row_means.restype = i32
+    L.rt_row_means.argtypes = [vp, vp, i32, u64, u64, ctypes.c_float, vp, vp]
+    L.rt_sr_copy.restype = i32
+    L.rt_sr_copy.argtypes = [vp, vp, u64, vp, u64, vp]
+    L.rt_set_timing.restype = i32
+    L.rt_set_timing.argtypes = [vp, i32]
+    L.rt_last_kernel_ms.restype = i32
+    L.rt_last_kernel_ms.argtypes = [vp, ctypes.POINTER(ctypes.c_float)]
+    L.rt_streamed_stats.restype = i32
+    L.rt_streamed_stats.argtypes = [vp, ctypes.POINTER(ctypes.c_double)]
+    v = L.rt_version()
+    if v != ABI_VERSION:
+        raise RuntimeError(f"{LIB_PATH} has ABI version {v}, this package expects {ABI_VERSION}; rebuild it")
+    _lib = L
+    return L
+
+
+def check(code: int) -> None:
+    if code != RT_OK:
+        raise NativeError(code, lib().rt_last_error().decode("utf-8", "replace"))
+
+
+class Handle:
+    """Owns one ``rt_handle`` (workspace of one device)."""
+
+    def __init__(self, device: int):
+        self._h = ctypes.c_void_p()
+        check(lib().rt_create(int(device), ctypes.byref(self._h)))
+        self.device = int(device)
+
+    @property
+    def ptr(self) -> ctypes.c_void_p:
+        if not self._h:
+            raise RuntimeError("handle already destroyed")
+        return self._h
+
+    def close(self) -> None:
+        if self._h:
+            lib().rt_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # -- thin wrappers ---------------------------------------------------------
+    def step_multi(self, descs, n, scalars, n_scalars, seed, noise_mode, d_clip_coef=None, d_skip=None, stream=0):
+        check(lib().rt_step_multi(self.ptr, descs, n, scalars, n_scalars, seed, noise_mode, d_clip_coef, d_skip,
+                                  stream))
+
+    def step_streamed(self, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, stream=0):
+        check(lib().rt_step_streamed(self.ptr, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, stream))
+
+    def grad_norm(self, descs, n, inv_loss_scale, max_norm, d_out, stream=0):
+        check(lib().rt_grad_norm(self.ptr, descs, n, inv_loss_scale, max_norm, d_out, stream))
+
+    def row_means(self, g, g_dtype, rows, row_len, inv_loss_scale, d_row_mean, stream=0):
+        check(lib().rt_row_means(self.ptr, g, g_dtype, rows, row_len, inv_loss_scale, d_row_mean, stream))
+
+    def set_timing(self, enabled: bool) -> None:
+        check(lib().rt_set_timing(self.ptr, int(enabled)))
+
+    def last_kernel_ms(self) -> float:
+        ms = ctypes.c_float()
+        check(lib().rt_last_kernel_ms(self.ptr, ctypes.byref(ms)))
+        return ms.value
+
+    def streamed_stats(self):
+        out = (ctypes.c_double * 3)()
+        check(lib().rt_streamed_stats(self.ptr, out))
+        return {"bytes_h2d": out[0], "bytes_d2h": out[1], "seconds": out[2]}
+
+
+def sr_copy(target_ptr, source_ptr, numel, noise_ptr, seed, stream=0) -> None:
+    check(lib().rt_sr_copy(target_ptr, source_ptr, numel, noise_ptr, seed, stream))

@@ -1,0 +1,725 @@
+// Host side of the C ABI declared in include/ramtorch_sr_adamw.h: argument
+// checks, the device-side tensor / chunk tables, kernel dispatch by dtype
+// combination, and the streamed (host-resident) pipeline.  gfx950 only.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <chrono>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <new>
+#include <vector>
+
+#include "kernels.h"
+
+using namespace rt;
+
+// ---------------------------------------------------------------------------
+// error reporting
+// ---------------------------------------------------------------------------
+static thread_local char g_err[512] = "";
+
+static int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                          \
+    do {                                                                                       \
+        hipError_t e_ = (expr);                                                                \
+        if (e_ != hipSuccess)                                                                  \
+            return fail(RT_EHIP, "%s failed: %s (%d) at %s:%d", #expr, hipGetErrorString(e_), \
+                        (int)e_, __FILE__, __LINE__);                                          \
+    } while (0)
+
+// ---------------------------------------------------------------------------
+// handle
+// ---------------------------------------------------------------------------
+namespace {
+
+constexpr int kSlots = 2;            // table staging slots (host runs at most this far ahead)
+constexpr int kNormPartials = 2048;  // workgroups of the norm pass
+
+struct DevBuf {
+    void* ptr = nullptr;
+    size_t cap = 0;
+};
+
+// One staging slot for the tables of one launch batch: pinned host image,
+// device copy, and an event recorded after the kernels that read the copy.
+struct TableSlot {
+    DevBuf dev;
+    void* host = nullptr;  // pinned; keeps the image last uploaded to `dev`
+    size_t host_cap = 0;
+    size_t valid_bytes = 0;  // bytes of `host` that `dev` currently mirrors
+    hipEvent_t done = nullptr;
+    bool in_flight = false;
+};
+
+struct Streamed {
+    hipStream_t h2d = nullptr, comp = nullptr, d2h = nullptr;
+    hipEvent_t start = nullptr;
+    hipEvent_t h2d_done[2] = {nullptr, nullptr};
+    hipEvent_t comp_done[2] = {nullptr, nullptr};
+    hipEvent_t d2h_done[2] = {nullptr, nullptr};
+    DevBuf stage[4][2];  // [p,g,m,v][buffer]
+    bool ready = false;
+    double bytes_h2d = 0, bytes_d2h = 0, seconds = 0;
+};
+
+}  // namespace
+
+struct rt_handle {
+    int device = 0;
+    TableSlot slots[kSlots];
+    uint64_t slot_counter = 0;
+    DevBuf norm_partials;
+    std::vector<uint8_t> image;  // scratch for building a table image
+    bool timing = false;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    bool timed = false;
+    Streamed st;
+};
+
+static int dev_reserve(DevBuf& b, size_t bytes) {
+    if (bytes <= b.cap) return RT_OK;
+    if (b.ptr) {
+        HIP_TRY(hipFree(b.ptr));
+        b.ptr = nullptr;
+        b.cap = 0;
+    }
+    size_t want = std::max(bytes + bytes / 4, (size_t)4096);
+    hipError_t e = hipMalloc(&b.ptr, want);
+    if (e != hipSuccess) {
+        b.ptr = nullptr;
+        return fail(RT_ENOMEM, "hipMalloc(%zu) failed: %s", want, hipGetErrorString(e));
+    }
+    b.cap = want;
+    return RT_OK;
+}
+
+static int dtype_size(int dt) { return dt == RT_DT_F32 ? 4 : 2; }
+
+// ---------------------------------------------------------------------------
+// kernel dispatch
+// ---------------------------------------------------------------------------
+using MultiKernel = void (*)(const DevTensor*, const ChunkRef*, const DevScalars*, uint32_t, uint32_t,
+                             const float*, const uint32_t*);
+
+template <int P, int G, int M, int V>
+static MultiKernel pick_noise(int noise) {
+    return noise == RT_NOISE_EXPLICIT ? sr_adamw_multi_kernel<P, G, M, V, RT_NOISE_EXPLICIT>
+                                      : sr_adamw_multi_kernel<P, G, M, V, RT_NOISE_PHILOX>;
+}
+template <int P, int G, int M>
+static MultiKernel pick_v(int v, int noise) {
+    return v == RT_DT_BF16 ? pick_noise<P, G, M, RT_DT_BF16>(noise) : pick_noise<P, G, M, RT_DT_F32>(noise);
+}
+template <int P, int G>
+static MultiKernel pick_m(int m, int v, int noise) {
+    return m == RT_DT_BF16 ? pick_v<P, G, RT_DT_BF16>(v, noise) : pick_v<P, G, RT_DT_F32>(v, noise);
+}
+template <int P>
+static MultiKernel pick_g(int g, int m, int v, int noise) {
+    switch (g) {
+        case RT_DT_BF16: return pick_m<P, RT_DT_BF16>(m, v, noise);
+        case RT_DT_F32: return pick_m<P, RT_DT_F32>(m, v, noise);
+        default: return pick_m<P, RT_DT_F16>(m, v, noise);
+    }
+}
+static MultiKernel pick_kernel(int p, int g, int m, int v, int noise) {
+    return p == RT_DT_BF16 ? pick_g<RT_DT_BF16>(g, m, v, noise) : pick_g<RT_DT_F32>(g, m, v, noise);
+}
+
+static inline uint32_t combo_of(const rt_tensor_desc& d) {
+    return (uint32_t)d.p_dtype | ((uint32_t)d.g_dtype << 2) | ((uint32_t)d.m_dtype << 4) |
+           ((uint32_t)d.v_dtype << 6);
+}
+
+// ---------------------------------------------------------------------------
+// argument validation shared by the resident and streamed entry points
+// ---------------------------------------------------------------------------
+static int validate(const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars, uint32_t n_scalars,
+                    int noise_mode, bool allow_host) {
+    if (n > 0 && descs == nullptr) return fail(RT_EINVAL, "descs is NULL with n=%u", n);
+    if (n > 0 && (scalars == nullptr || n_scalars == 0)) return fail(RT_EINVAL, "scalars missing");
+    if (noise_mode != RT_NOISE_PHILOX && noise_mode != RT_NOISE_EXPLICIT)
+        return fail(RT_EINVAL, "unknown noise_mode %d", noise_mode);
+    for (uint32_t i = 0; i < n; ++i) {
+        const rt_tensor_desc& d = descs[i];
+        if (d.p_dtype != RT_DT_BF16 && d.p_dtype != RT_DT_F32)
+            return fail(RT_EUNSUPPORTED, "tensor %u: p_dtype %d (need bf16 or f32)", i, d.p_dtype);
+        if (d.m_dtype != RT_DT_BF16 && d.m_dtype != RT_DT_F32)
+            return fail(RT_EUNSUPPORTED, "tensor %u: m_dtype %d (need bf16 or f32)", i, d.m_dtype);
+        if (d.v_dtype != RT_DT_BF16 && d.v_dtype != RT_DT_F32)
+            return fail(RT_EUNSUPPORTED, "tensor %u: v_dtype %d (need bf16 or f32)", i, d.v_dtype);
+        if (d.g_dtype > RT_DT_F16) return fail(RT_EINVAL, "tensor %u: g_dtype %d unknown", i, d.g_dtype);
+        if (d.scalars_idx >= n_scalars)
+            return fail(RT_EINVAL, "tensor %u: scalars_idx %u >= %u", i, d.scalars_idx, n_scalars);
+        if (d.tensor_id >= (1u << 30)) return fail(RT_EINVAL, "tensor %u: tensor_id %u >= 2^30", i, d.tensor_id);
+        if (d.elem_offset & 7u)
+            return fail(RT_EINVAL, "tensor %u: elem_offset %llu not a multiple of 8", i,
+                        (unsigned long long)d.elem_offset);
+        if (!allow_host && d.host_mask != 0)
+            return fail(RT_EINVAL, "tensor %u: host_mask set on the resident entry point", i);
+        if (d.numel == 0) continue;
+        if (!d.p || !d.g || !d.m || !d.v) return fail(RT_EINVAL, "tensor %u: NULL array pointer", i);
+        if (((uintptr_t)d.p % dtype_size(d.p_dtype)) || ((uintptr_t)d.g % dtype_size(d.g_dtype)) ||
+            ((uintptr_t)d.m % dtype_size(d.m_dtype)) || ((uintptr_t)d.v % dtype_size(d.v_dtype)))
+            return fail(RT_EINVAL, "tensor %u: array pointer not aligned to its element size", i);
+        if (d.numel / kChunkElems >= 0xFFFFFFFFull)
+            return fail(RT_EUNSUPPORTED, "tensor %u: numel %llu too large", i, (unsigned long long)d.numel);
+        if (noise_mode == RT_NOISE_EXPLICIT) {
+            if ((d.p_dtype == RT_DT_BF16 && !d.noise_p) || (d.m_dtype == RT_DT_BF16 && !d.noise_m) ||
+                (d.v_dtype == RT_DT_BF16 && !d.noise_v))
+                return fail(RT_EINVAL, "tensor %u: explicit noise missing for a bf16 array", i);
+        }
+        if (scalars[d.scalars_idx].centralization != 0.0f) {
+            if (!d.row_mean || d.row_len == 0)
+                return fail(RT_EINVAL, "tensor %u: centralization without row_mean/row_len", i);
+        }
+    }
+    return RT_OK;
+}
+
+// ---------------------------------------------------------------------------
+// table building and launch
+// ---------------------------------------------------------------------------
+namespace {
+
+struct Batch {            // tensors of one dtype combination inside a table image
+    uint32_t combo;
+    uint32_t first_chunk;
+    uint32_t n_chunks;
+};
+
+struct Plan {
+    size_t off_sets = 0, off_tensors = 0, off_chunks = 0, off_gdt = 0, bytes = 0;
+    uint32_t n_sets = 0, n_tensors = 0, n_chunks = 0;
+    std::vector<Batch> batches;
+};
+
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+}  // namespace
+
+// Lays out [DevScalars sets][DevTensor records][ChunkRef list][g dtype bytes]
+// in h->image.  Tensors are grouped by dtype combination so that each
+// combination is one contiguous chunk range = one launch.
+static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
+                        bool want_explicit, Plan& plan) {
+    // (scalars_idx, step) -> set index
+    std::map<std::pair<uint32_t, uint32_t>, uint32_t> set_of;
+    std::vector<DevScalars> sets;
+    std::vector<uint32_t> order;
+    order.reserve(n);
+    for (uint32_t i = 0; i < n; ++i)
+        if (descs[i].numel != 0) order.push_back(i);
+    std::stable_sort(order.begin(), order.end(),
+                     [&](uint32_t a, uint32_t b) { return combo_of(descs[a]) < combo_of(descs[b]); });
+
+    std::vector<DevTensor> tens(order.size());
+    uint64_t total_chunks = 0;
+    for (size_t k = 0; k < order.size(); ++k) {
+        const rt_tensor_desc& d = descs[order[k]];
+        auto key = std::make_pair(d.scalars_idx, d.step);
+        auto it = set_of.find(key);
+        if (it == set_of.end()) {
+            DevScalars ds;
+            memset(&ds, 0, sizeof(ds));
+            ds.s = scalars[d.scalars_idx];
+            ds.step = d.step;
+            it = set_of.emplace(key, (uint32_t)sets.size()).first;
+            sets.push_back(ds);
+        }
+        DevTensor& t = tens[k];
+        memset(&t, 0, sizeof(t));
+        t.p = (uint64_t)d.p; t.g = (uint64_t)d.g; t.m = (uint64_t)d.m; t.v = (uint64_t)d.v;
+        if (want_explicit) {
+            t.np = (uint64_t)d.noise_p; t.nm = (uint64_t)d.noise_m; t.nv = (uint64_t)d.noise_v;
+        }
+        t.dp = (uint64_t)d.dbg_p; t.dm = (uint64_t)d.dbg_m; t.dv = (uint64_t)d.dbg_v;
+        t.row_mean = sets[it->second].s.centralization != 0.0f ? (uint64_t)d.row_mean : 0;
+        t.numel = d.numel;
+        t.block_base = d.elem_offset >> 3;
+        t.row_len = d.row_len ? d.row_len : 1;
+        t.tensor_id4 = d.tensor_id * 4u;
+        t.set_idx = it->second;
+        const uint64_t all = t.p | t.g | t.m | t.v | t.np | t.nm | t.nv;
+        t.flags = (all & 15u) == 0 ? kFlagAligned : 0u;
+        total_chunks += (d.numel + kChunkElems - 1) / kChunkElems;
+    }
+
+    plan.n_sets = (uint32_t)sets.size();
+    plan.n_tensors = (uint32_t)tens.size();
+    plan.n_chunks = (uint32_t)total_chunks;
+    plan.off_sets = 0;
+    plan.off_tensors = align_up(sets.size() * sizeof(DevScalars), 128);
+    plan.off_chunks = plan.off_tensors + align_up(tens.size() * sizeof(DevTensor), 128);
+    plan.off_gdt = plan.off_chunks + align_up(total_chunks * sizeof(ChunkRef), 128);
+    plan.bytes = plan.off_gdt + align_up(tens.size(), 128);
+    h->image.assign(plan.bytes, 0);
+    uint8_t* img = h->image.data();
+    if (!sets.empty()) memcpy(img + plan.off_sets, sets.data(), sets.size() * sizeof(DevScalars));
+    if (!tens.empty()) memcpy(img + plan.off_tensors, tens.data(), tens.size() * sizeof(DevTensor));
+    ChunkRef* cr = (ChunkRef*)(img + plan.off_chunks);
+    uint8_t* gdt = img + plan.off_gdt;
+    uint32_t c = 0;
+    plan.batches.clear();
+    for (size_t k = 0; k < order.size(); ++k) {
+        const rt_tensor_desc& d = descs[order[k]];
+        const uint32_t combo = combo_of(d);
+        if (plan.batches.empty() || plan.batches.back().combo != combo) plan.batches.push_back({combo, c, 0});
+        const uint32_t nc = (uint32_t)((d.numel + kChunkElems - 1) / kChunkElems);
+        for (uint32_t j = 0; j < nc; ++j) cr[c++] = ChunkRef{(uint32_t)k, j};
+        plan.batches.back().n_chunks += nc;
+        gdt[k] = d.g_dtype;
+    }
+}
+
+// Puts h->image into a free table slot (skipping the copy when the slot's
+// device memory already holds the same bytes) and returns the slot.
+static int stage_image(rt_handle* h, const Plan& plan, hipStream_t stream, TableSlot** out) {
+    TableSlot& s = h->slots[h->slot_counter++ % kSlots];
+    if (s.in_flight) {
+        HIP_TRY(hipEventSynchronize(s.done));
+        s.in_flight = false;
+    }
+    if (plan.bytes > s.host_cap) {
+        if (s.host) HIP_TRY(hipHostFree(s.host));
+        s.host = nullptr;
+        s.host_cap = 0;
+        s.valid_bytes = 0;
+        const size_t want = plan.bytes + plan.bytes / 4 + 4096;
+        hipError_t e = hipHostMalloc(&s.host, want, hipHostMallocDefault);
+        if (e != hipSuccess) return fail(RT_ENOMEM, "hipHostMalloc(%zu) failed: %s", want, hipGetErrorString(e));
+        s.host_cap = want;
+    }
+    if (plan.bytes > s.dev.cap) {
+        s.valid_bytes = 0;
+        int rc = dev_reserve(s.dev, plan.bytes);
+        if (rc != RT_OK) return rc;
+    }
+    const bool same = s.valid_bytes == plan.bytes && memcmp(s.host, h->image.data(), plan.bytes) == 0;
+    if (!same && plan.bytes > 0) {
+        memcpy(s.host, h->image.data(), plan.bytes);
+        HIP_TRY(hipMemcpyAsync(s.dev.ptr, s.host, plan.bytes, hipMemcpyHostToDevice, stream));
+        s.valid_bytes = plan.bytes;
+    }
+    *out = &s;
+    return RT_OK;
+}
+
+static int launch_update(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
+                         uint64_t seed, int noise_mode, const float* d_clip_coef, const uint32_t* d_skip,
+                         hipStream_t stream) {
+    Plan plan;
+    build_image(h, descs, n, scalars, noise_mode == RT_NOISE_EXPLICIT, plan);
+    if (plan.n_chunks == 0) return RT_OK;
+    TableSlot* slot = nullptr;
+    int rc = stage_image(h, plan, stream, &slot);
+    if (rc != RT_OK) return rc;
+    const uint8_t* base = (const uint8_t*)slot->dev.ptr;
+    const DevScalars* sets = (const DevScalars*)(base + plan.off_sets);
+    const DevTensor* tens = (const DevTensor*)(base + plan.off_tensors);
+    const ChunkRef* chunks = (const ChunkRef*)(base + plan.off_chunks);
+    if (h->timing) HIP_TRY(hipEventRecord(h->t0, stream));
+    for (const Batch& b : plan.batches) {
+        MultiKernel k = pick_kernel(b.combo & 3, (b.combo >> 2) & 3, (b.combo >> 4) & 3, (b.combo >> 6) & 3,
+                                    noise_mode);
+        hipLaunchKernelGGL(k, dim3(b.n_chunks), dim3(kThreads), 0, stream, tens, chunks + b.first_chunk, sets,
+                           (uint32_t)seed, (uint32_t)(seed >> 32), d_clip_coef, d_skip);
+        HIP_TRY(hipGetLastError());
+    }
+    if (h->timing) {
+        HIP_TRY(hipEventRecord(h->t1, stream));
+        h->timed = true;
+    }
+    HIP_TRY(hipEventRecord(slot->done, stream));
+    slot->in_flight = true;
+    return RT_OK;
+}
+
+// ---------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------
+extern "C" {
+
+int rt_version(void) { return RT_ABI_VERSION; }
+
+const char* rt_last_error(void) { return g_err; }
+
+int rt_create(int device, rt_handle** out) {
+    if (!out) return fail(RT_EINVAL, "out is NULL");
+    *out = nullptr;
+    int count = 0;
+    HIP_TRY(hipGetDeviceCount(&count));
+    if (device < 0 || device >= count) return fail(RT_EINVAL, "device %d out of range (have %d)", device, count);
+    HIP_TRY(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(RT_EUNSUPPORTED, "device %d is %s; this library is built for gfx950 only", device,
+                    prop.gcnArchName);
+    rt_handle* h = new (std::nothrow) rt_handle();
+    if (!h) return fail(RT_ENOMEM, "out of host memory");
+    h->device = device;
+    for (int i = 0; i < kSlots; ++i) HIP_TRY(hipEventCreateWithFlags(&h->slots[i].done, hipEventDisableTiming));
+    HIP_TRY(hipEventCreate(&h->t0));
+    HIP_TRY(hipEventCreate(&h->t1));
+    *out = h;
+    return RT_OK;
+}
+
+int rt_destroy(rt_handle* h) {
+    if (!h) return RT_OK;
+    (void)hipSetDevice(h->device);
+    (void)hipDeviceSynchronize();
+    for (int i = 0; i < kSlots; ++i) {
+        if (h->slots[i].dev.ptr) (void)hipFree(h->slots[i].dev.ptr);
+        if (h->slots[i].host) (void)hipHostFree(h->slots[i].host);
+        if (h->slots[i].done) (void)hipEventDestroy(h->slots[i].done);
+    }
+    if (h->norm_partials.ptr) (void)hipFree(h->norm_partials.ptr);
+    if (h->t0) (void)hipEventDestroy(h->t0);
+    if (h->t1) (void)hipEventDestroy(h->t1);
+    Streamed& st = h->st;
+    for (int a = 0; a < 4; ++a)
+        for (int b = 0; b < 2; ++b)
+            if (st.stage[a][b].ptr) (void)hipFree(st.stage[a][b].ptr);
+    for (int b = 0; b < 2; ++b) {
+        if (st.h2d_done[b]) (void)hipEventDestroy(st.h2d_done[b]);
+        if (st.comp_done[b]) (void)hipEventDestroy(st.comp_done[b]);
+        if (st.d2h_done[b]) (void)hipEventDestroy(st.d2h_done[b]);
+    }
+    if (st.start) (void)hipEventDestroy(st.start);
+    if (st.h2d) (void)hipStreamDestroy(st.h2d);
+    if (st.comp) (void)hipStreamDestroy(st.comp);
+    if (st.d2h) (void)hipStreamDestroy(st.d2h);
+    delete h;
+    return RT_OK;
+}
+
+int rt_set_timing(rt_handle* h, int enabled) {
+    if (!h) return fail(RT_EINVAL, "handle is NULL");
+    h->timing = enabled != 0;
+    h->timed = false;
+    return RT_OK;
+}
+
+int rt_last_kernel_ms(rt_handle* h, float* ms) {
+    if (!h || !ms) return fail(RT_EINVAL, "NULL argument");
+    if (!h->timed) return fail(RT_EINVAL, "no timed launch on this handle (rt_set_timing first)");
+    HIP_TRY(hipEventSynchronize(h->t1));
+    HIP_TRY(hipEventElapsedTime(ms, h->t0, h->t1));
+    return RT_OK;
+}
+
+int rt_step_multi(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
+                  uint32_t n_scalars, uint64_t seed, int noise_mode, const float* d_clip_coef,
+                  const uint32_t* d_skip, void* stream) {
+    if (!h) return fail(RT_EINVAL, "handle is NULL");
+    int rc = validate(descs, n, scalars, n_scalars, noise_mode, /*allow_host=*/false);
+    if (rc != RT_OK) return rc;
+    if (n == 0) return RT_OK;
+    HIP_TRY(hipSetDevice(h->device));
+    return launch_update(h, descs, n, scalars, seed, noise_mode, d_clip_coef, d_skip, (hipStream_t)stream);
+}
+
+int rt_grad_norm(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, float inv_loss_scale, float max_norm,
+                 void* d_out, void* stream_) {
+    if (!h) return fail(RT_EINVAL, "handle is NULL");
+    if (!d_out || ((uintptr_t)d_out & 15u)) return fail(RT_EINVAL, "d_out must be a 16-byte aligned device pointer");
+    if (n > 0 && !descs) return fail(RT_EINVAL, "descs is NULL");
+    hipStream_t stream = (hipStream_t)stream_;
+    HIP_TRY(hipSetDevice(h->device));
+    // Reuse the table builder with a descriptor copy that only carries g.
+    std::vector<rt_tensor_desc> gd(descs, descs + n);
+    rt_scalars one;
+    memset(&one, 0, sizeof(one));
+    one.inv_loss_scale = 1.0f;
+    for (uint32_t i = 0; i < n; ++i) {
+        rt_tensor_desc& d = gd[i];
+        if (d.g_dtype > RT_DT_F16) return fail(RT_EINVAL, "tensor %u: g_dtype %d unknown", i, d.g_dtype);
+        if (d.numel && !d.g) return fail(RT_EINVAL, "tensor %u: g is NULL", i);
+        if (d.numel && ((uintptr_t)d.g % dtype_size(d.g_dtype)))
+            return fail(RT_EINVAL, "tensor %u: g not aligned to its element size", i);
+        if (d.numel / kChunkElems >= 0xFFFFFFFFull) return fail(RT_EUNSUPPORTED, "tensor %u: numel too large", i);
+        if (d.host_mask) return fail(RT_EINVAL, "tensor %u: host_mask set (grads must be device resident)", i);
+        d.p = d.m = d.v = nullptr;
+        d.noise_p = d.noise_m = d.noise_v = nullptr;
+        d.dbg_p = d.dbg_m = d.dbg_v = nullptr;
+        d.row_mean = nullptr;
+        d.scalars_idx = 0;
+        d.step = 0;
+        d.elem_offset = 0;
+        // one dtype combination => one chunk list; the real gradient dtype is looked up per tensor
+        d.p_dtype = d.g_dtype = d.m_dtype = d.v_dtype = RT_DT_BF16;
+    }
+    Plan plan;
+    build_image(h, gd.data(), n, &one, false, plan);
+    {
+        // build_image keeps the input order inside one combination
+        uint8_t* gdt = h->image.data() + plan.off_gdt;
+        uint32_t k = 0;
+        for (uint32_t i = 0; i < n; ++i)
+            if (descs[i].numel != 0) gdt[k++] = descs[i].g_dtype;
+    }
+    int rc = dev_reserve(h->norm_partials, kNormPartials * sizeof(double));
+    if (rc != RT_OK) return rc;
+    uint32_t grid = std::min<uint32_t>(kNormPartials, std::max<uint32_t>(plan.n_chunks, 1u));
+    if (plan.n_chunks == 0) {
+        HIP_TRY(hipMemsetAsync(h->norm_partials.ptr, 0, sizeof(double), stream));
+        grid = 1;
+    } else {
+        TableSlot* slot = nullptr;
+        rc = stage_image(h, plan, stream, &slot);
+        if (rc != RT_OK) return rc;
+        const uint8_t* base = (const uint8_t*)slot->dev.ptr;
+        hipLaunchKernelGGL(grad_sumsq_kernel, dim3(grid), dim3(kThreads), 0, stream,
+                           (const DevTensor*)(base + plan.off_tensors), (const ChunkRef*)(base + plan.off_chunks),
+                           plan.n_chunks, base + plan.off_gdt, inv_loss_scale, (double*)h->norm_partials.ptr);
+        HIP_TRY(hipGetLastError());
+        HIP_TRY(hipEventRecord(slot->done, stream));
+        slot->in_flight = true;
+    }
+    hipLaunchKernelGGL(grad_norm_finish_kernel, dim3(1), dim3(kThreads), 0, stream,
+                       (const double*)h->norm_partials.ptr, grid, max_norm, (float*)d_out);
+    HIP_TRY(hipGetLastError());
+    return RT_OK;
+}
+
+int rt_row_means(rt_handle* h, const void* g, int g_dtype, uint64_t rows, uint64_t row_len, float inv_loss_scale,
+                 float* d_row_mean, void* stream_) {
+    if (!h) return fail(RT_EINVAL, "handle is NULL");
+    if (rows == 0) return RT_OK;
+    if (!g || !d_row_mean || row_len == 0) return fail(RT_EINVAL, "NULL pointer or empty row");
+    if (rows > 0x7FFFFFFFull) return fail(RT_EUNSUPPORTED, "too many rows");
+    hipStream_t stream = (hipStream_t)stream_;
+    HIP_TRY(hipSetDevice(h->device));
+    switch (g_dtype) {
+        case RT_DT_BF16:
+            hipLaunchKernelGGL(row_mean_kernel<RT_DT_BF16>, dim3((uint32_t)rows), dim3(kThreads), 0, stream,
+                               (uint64_t)g, row_len, inv_loss_scale, d_row_mean);
+            break;
+        case RT_DT_F32:
+            hipLaunchKernelGGL(row_mean_kernel<RT_DT_F32>, dim3((uint32_t)rows), dim3(kThreads), 0, stream,
+                               (uint64_t)g, row_len, inv_loss_scale, d_row_mean);
+            break;
+        case RT_DT_F16:
+            hipLaunchKernelGGL(row_mean_kernel<RT_DT_F16>, dim3((uint32_t)rows), dim3(kThreads), 0, stream,
+                               (uint64_t)g, row_len, inv_loss_scale, d_row_mean);
+            break;
+        default: return fail(RT_EINVAL, "g_dtype %d unknown", g_dtype);
+    }
+    HIP_TRY(hipGetLastError());
+    return RT_OK;
+}
+
+int rt_sr_copy(void* target_bf16, const float* source, uint64_t numel, const void* noise, uint64_t seed,
+               void* stream_) {
+    if (numel == 0) return RT_OK;
+    if (!target_bf16 || !source) return fail(RT_EINVAL, "NULL pointer");
+    if (((uintptr_t)target_bf16 & 1u) || ((uintptr_t)source & 3u) || ((uintptr_t)noise & 1u))
+        return fail(RT_EINVAL, "pointer not aligned to its element size");
+    hipStream_t stream = (hipStream_t)stream_;
+    const int aligned = ((((uintptr_t)target_bf16) | ((uintptr_t)source) | ((uintptr_t)noise)) & 15u) == 0;
+    const uint64_t vecs = (numel + kVec - 1) / kVec;
+    const uint32_t grid = (uint32_t)std::min<uint64_t>((vecs + kThreads - 1) / kThreads, 256u * 16u);
+    if (noise)
+        hipLaunchKernelGGL(sr_copy_kernel<RT_NOISE_EXPLICIT>, dim3(grid), dim3(kThreads), 0, stream,
+                           (uint64_t)target_bf16, (uint64_t)source, numel, (uint64_t)noise, (uint32_t)seed,
+                           (uint32_t)(seed >> 32), aligned);
+    else
+        hipLaunchKernelGGL(sr_copy_kernel<RT_NOISE_PHILOX>, dim3(grid), dim3(kThreads), 0, stream,
+                           (uint64_t)target_bf16, (uint64_t)source, numel, (uint64_t)0, (uint32_t)seed,
+                           (uint32_t)(seed >> 32), aligned);
+    HIP_TRY(hipGetLastError());
+    return RT_OK;
+}
+
+// ---------------------------------------------------------------------------
+// streamed variant
+// ---------------------------------------------------------------------------
+static int streamed_init(rt_handle* h) {
+    Streamed& st = h->st;
+    if (st.ready) return RT_OK;
+    HIP_TRY(hipStreamCreateWithFlags(&st.h2d, hipStreamNonBlocking));
+    HIP_TRY(hipStreamCreateWithFlags(&st.comp, hipStreamNonBlocking));
+    HIP_TRY(hipStreamCreateWithFlags(&st.d2h, hipStreamNonBlocking));
+    HIP_TRY(hipEventCreateWithFlags(&st.start, hipEventDisableTiming));
+    for (int b = 0; b < 2; ++b) {
+        HIP_TRY(hipEventCreateWithFlags(&st.h2d_done[b], hipEventDisableTiming));
+        HIP_TRY(hipEventCreateWithFlags(&st.comp_done[b], hipEventDisableTiming));
+        HIP_TRY(hipEventCreateWithFlags(&st.d2h_done[b], hipEventDisableTiming));
+    }
+    st.ready = true;
+    return RT_OK;
+}
+
+namespace {
+struct Segment {       // a contiguous piece of one tensor inside one chunk
+    uint32_t tensor;   // index into descs
+    uint64_t start;    // first element of the piece inside the tensor
+    uint64_t count;
+    uint64_t stage_off;  // element offset inside the staging buffers (multiple of 8)
+};
+}  // namespace
+
+int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
+                     uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems, void* stream_) {
+    if (!h) return fail(RT_EINVAL, "handle is NULL");
+    int rc = validate(descs, n, scalars, n_scalars, noise_mode, /*allow_host=*/true);
+    if (rc != RT_OK) return rc;
+    if (chunk_elems < kVec || (chunk_elems % kVec) != 0)
+        return fail(RT_EINVAL, "chunk_elems %llu must be a positive multiple of 8", (unsigned long long)chunk_elems);
+    if (noise_mode == RT_NOISE_EXPLICIT) {
+        // noise arrays are addressed per piece below; they must be device resident
+    }
+    for (uint32_t i = 0; i < n; ++i)
+        if (descs[i].row_mean && scalars[descs[i].scalars_idx].centralization != 0.0f && descs[i].row_len == 0)
+            return fail(RT_EINVAL, "tensor %u: row_len is 0", i);
+    if (n == 0) return RT_OK;
+    hipStream_t user = (hipStream_t)stream_;
+    HIP_TRY(hipSetDevice(h->device));
+    rc = streamed_init(h);
+    if (rc != RT_OK) return rc;
+    Streamed& st = h->st;
+    const auto wall0 = std::chrono::steady_clock::now();
+
+    // ---- cut the tensor list into chunks of at most chunk_elems staged elements
+    std::vector<std::vector<Segment>> chunks;
+    {
+        std::vector<Segment> cur;
+        uint64_t used = 0;
+        for (uint32_t i = 0; i < n; ++i) {
+            uint64_t done = 0;
+            const uint64_t numel = descs[i].numel;
+            while (done < numel) {
+                if (used >= chunk_elems) {
+                    chunks.push_back(std::move(cur));
+                    cur.clear();
+                    used = 0;
+                }
+                const uint64_t take = std::min(numel - done, chunk_elems - used);
+                cur.push_back(Segment{i, done, take, used});
+                done += take;
+                used = align_up(used + take, kVec);  // next piece starts 16-byte aligned
+            }
+        }
+        if (!cur.empty()) chunks.push_back(std::move(cur));
+    }
+
+    // ---- staging buffers sized for the widest element type that is host resident
+    int stage_esize[4] = {0, 0, 0, 0};
+    for (uint32_t i = 0; i < n; ++i) {
+        const rt_tensor_desc& d = descs[i];
+        if (d.numel == 0) continue;
+        if (d.host_mask & RT_HOST_P) stage_esize[0] = std::max(stage_esize[0], dtype_size(d.p_dtype));
+        if (d.host_mask & RT_HOST_G) stage_esize[1] = std::max(stage_esize[1], dtype_size(d.g_dtype));
+        if (d.host_mask & RT_HOST_M) stage_esize[2] = std::max(stage_esize[2], dtype_size(d.m_dtype));
+        if (d.host_mask & RT_HOST_V) stage_esize[3] = std::max(stage_esize[3], dtype_size(d.v_dtype));
+    }
+    uint64_t max_used = 0;
+    for (const auto& c : chunks)
+        if (!c.empty()) max_used = std::max(max_used, align_up(c.back().stage_off + c.back().count, kVec));
+    for (int a = 0; a < 4; ++a)
+        for (int b = 0; b < 2; ++b)
+            if (stage_esize[a]) {
+                rc = dev_reserve(st.stage[a][b], max_used * 4);  // sized for fp32 so dtype changes never realloc
+                if (rc != RT_OK) return rc;
+            }
+
+    // grads (and anything else already queued by the caller) must be ready
+    HIP_TRY(hipEventRecord(st.start, user));
+    HIP_TRY(hipStreamWaitEvent(st.h2d, st.start, 0));
+    HIP_TRY(hipStreamWaitEvent(st.comp, st.start, 0));
+
+    st.bytes_h2d = st.bytes_d2h = 0;
+    std::vector<rt_tensor_desc> piece;
+    bool used_buf[2] = {false, false};
+    for (size_t c = 0; c < chunks.size(); ++c) {
+        const int b = (int)(c & 1);
+        const auto& segs = chunks[c];
+        // H2D: the buffer is free once the D2H of the chunk two back has finished
+        if (used_buf[b]) HIP_TRY(hipStreamWaitEvent(st.h2d, st.d2h_done[b], 0));
+        piece.clear();
+        for (const Segment& s : segs) {
+            const rt_tensor_desc& d = descs[s.tensor];
+            rt_tensor_desc q = d;
+            q.numel = s.count;
+            q.elem_offset = d.elem_offset + s.start;
+            q.host_mask = 0;
+            const int es[4] = {dtype_size(d.p_dtype), dtype_size(d.g_dtype), dtype_size(d.m_dtype),
+                               dtype_size(d.v_dtype)};
+            const void* src[4] = {d.p, d.g, d.m, d.v};
+            void* dst[4];
+            for (int a = 0; a < 4; ++a) {
+                if (d.host_mask & (1u << a)) {
+                    dst[a] = (uint8_t*)st.stage[a][b].ptr + s.stage_off * es[a];
+                    const size_t bytes = s.count * es[a];
+                    HIP_TRY(hipMemcpyAsync(dst[a], (const uint8_t*)src[a] + s.start * es[a], bytes,
+                                           hipMemcpyHostToDevice, st.h2d));
+                    st.bytes_h2d += (double)bytes;
+                } else {
+                    dst[a] = (uint8_t*)src[a] + s.start * es[a];
+                }
+            }
+            q.p = dst[0]; q.g = dst[1]; q.m = dst[2]; q.v = dst[3];
+            if (d.noise_p) q.noise_p = (const uint8_t*)d.noise_p + s.start * 2;
+            if (d.noise_m) q.noise_m = (const uint8_t*)d.noise_m + s.start * 2;
+            if (d.noise_v) q.noise_v = (const uint8_t*)d.noise_v + s.start * 2;
+            if (d.dbg_p) q.dbg_p = d.dbg_p + s.start;
+            if (d.dbg_m) q.dbg_m = d.dbg_m + s.start;
+            if (d.dbg_v) q.dbg_v = d.dbg_v + s.start;
+            piece.push_back(q);
+        }
+        HIP_TRY(hipEventRecord(st.h2d_done[b], st.h2d));
+
+        // compute
+        HIP_TRY(hipStreamWaitEvent(st.comp, st.h2d_done[b], 0));
+        rc = launch_update(h, piece.data(), (uint32_t)piece.size(), scalars, seed, noise_mode, nullptr, nullptr,
+                           st.comp);
+        if (rc != RT_OK) return rc;
+        HIP_TRY(hipEventRecord(st.comp_done[b], st.comp));
+
+        // D2H of the updated host-resident arrays (p, m, v; grads are read-only)
+        HIP_TRY(hipStreamWaitEvent(st.d2h, st.comp_done[b], 0));
+        for (size_t k = 0; k < segs.size(); ++k) {
+            const Segment& s = segs[k];
+            const rt_tensor_desc& d = descs[s.tensor];
+            const int es[4] = {dtype_size(d.p_dtype), 0, dtype_size(d.m_dtype), dtype_size(d.v_dtype)};
+            void* host[4] = {d.p, nullptr, d.m, d.v};
+            const void* dev[4] = {piece[k].p, nullptr, piece[k].m, piece[k].v};
+            for (int a = 0; a < 4; ++a) {
+                if (a == 1 || !(d.host_mask & (1u << a))) continue;
+                const size_t bytes = s.count * es[a];
+                HIP_TRY(hipMemcpyAsync((uint8_t*)host[a] + s.start * es[a], dev[a], bytes, hipMemcpyDeviceToHost,
+                                       st.d2h));
+                st.bytes_d2h += (double)bytes;
+            }
+        }
+        HIP_TRY(hipEventRecord(st.d2h_done[b], st.d2h));
+        used_buf[b] = true;
+    }
+    // Host memory is final on return; device-resident arrays are final for the caller's stream.
+    HIP_TRY(hipStreamSynchronize(st.d2h));
+    HIP_TRY(hipStreamSynchronize(st.comp));
+    st.seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - wall0).count();
+    return RT_OK;
+}
+
+int rt_streamed_stats(rt_handle* h, double out[3]) {
+    if (!h || !out) return fail(RT_EINVAL, "NULL argument");
+    out[0] = h->st.bytes_h2d;
+    out[1] = h->st.bytes_d2h;
+    out[2] = h->st.seconds;
+    return RT_OK;
+}
+
+}  // extern "C"

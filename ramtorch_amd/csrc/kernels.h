@@ -1,0 +1,526 @@
+// Device code of the stochastic-rounding AdamW step for gfx950 (wave64).
+//
+// The step is HBM-bound (14 bytes and ~25 flops per all-bf16 element), so the
+// kernels are plain vector code: 128-bit global loads and stores, fp32 math in
+// registers, a counter-based Philox4x32-10 for the rounding noise.  No LDS and
+// no MFMA in the update; wavefront reductions only in the norm / row-mean passes.
+//
+// Floating-point contraction is switched off for the whole file: the rounding
+// sequence of every operation is part of the contract (it has to reproduce
+// torch's GPU kernels bit for bit), so each fused multiply-add below is an
+// explicit __builtin_fmaf and nothing else may fuse.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "device_types.h"
+
+#pragma clang fp contract(off)
+
+namespace rt {
+
+// Every tensor pointer arrives as a 64-bit integer from a table; telling the
+// compiler it is global memory (address space 1) yields global_load/store
+// instead of flat accesses.
+#define RT_GLOBAL __attribute__((address_space(1)))
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+__device__ __forceinline__ u32x4 ldg128(uint64_t addr) { return *(const RT_GLOBAL u32x4*)addr; }
+__device__ __forceinline__ void stg128(uint64_t addr, u32x4 v) { *(RT_GLOBAL u32x4*)addr = v; }
+__device__ __forceinline__ uint32_t ldg16(uint64_t addr) { return *(const RT_GLOBAL uint16_t*)addr; }
+__device__ __forceinline__ void stg16(uint64_t addr, uint32_t v) { *(RT_GLOBAL uint16_t*)addr = (uint16_t)v; }
+__device__ __forceinline__ float ldg32f(uint64_t addr) { return *(const RT_GLOBAL float*)addr; }
+__device__ __forceinline__ void stg32f(uint64_t addr, float v) { *(RT_GLOBAL float*)addr = v; }
+
+template <int DT>
+__device__ __forceinline__ constexpr int esize() {
+    return DT == RT_DT_F32 ? 4 : 2;
+}
+
+// ---------------------------------------------------------------------------
+// Philox4x32-10 (Salmon et al. 2011).  The key schedule is wave-uniform (the
+// key is the seed), so the per-round key bumps stay in scalar registers.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ u32x4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
+                                               uint32_t k1) {
+    constexpr uint32_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u;
+    constexpr uint32_t W0 = 0x9E3779B9u, W1 = 0xBB67AE85u;
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        const uint64_t p0 = (uint64_t)M0 * c0;
+        const uint64_t p1 = (uint64_t)M1 * c2;
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+        const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+        c1 = (uint32_t)p1;
+        c3 = (uint32_t)p0;
+        c0 = n0;
+        c2 = n2;
+        k0 += W0;
+        k1 += W1;
+    }
+    u32x4 r;
+    r.x = c0; r.y = c1; r.z = c2; r.w = c3;
+    return r;
+}
+
+// ---------------------------------------------------------------------------
+// Raw 8-element vectors: one 128-bit word for 16-bit types, two for fp32.
+// ---------------------------------------------------------------------------
+template <int DT>
+struct Raw8 {
+    u32x4 a;
+    u32x4 b;  // used by fp32 only
+};
+
+template <int DT>
+__device__ __forceinline__ Raw8<DT> load_raw(uint64_t base, uint64_t i) {
+    Raw8<DT> r;
+    const uint64_t addr = base + i * esize<DT>();
+    r.a = ldg128(addr);
+    if constexpr (DT == RT_DT_F32) r.b = ldg128(addr + 16);
+    return r;
+}
+
+// Per-element load for tails and unaligned tensors: elements at or past n read as 0.
+template <int DT>
+__device__ __forceinline__ Raw8<DT> load_raw_guarded(uint64_t base, uint64_t i, uint64_t n) {
+    Raw8<DT> r;
+    uint32_t w[8];
+    if constexpr (DT == RT_DT_F32) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) w[j] = (i + j < n) ? f2u(ldg32f(base + (i + j) * 4)) : 0u;
+        r.a.x = w[0]; r.a.y = w[1]; r.a.z = w[2]; r.a.w = w[3];
+        r.b.x = w[4]; r.b.y = w[5]; r.b.z = w[6]; r.b.w = w[7];
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t lo = (i + 2 * k < n) ? ldg16(base + (i + 2 * k) * 2) : 0u;
+            const uint32_t hi = (i + 2 * k + 1 < n) ? ldg16(base + (i + 2 * k + 1) * 2) : 0u;
+            w[k] = lo | (hi << 16);
+        }
+        r.a.x = w[0]; r.a.y = w[1]; r.a.z = w[2]; r.a.w = w[3];
+    }
+    return r;
+}
+
+template <int DT>
+__device__ __forceinline__ void decode(const Raw8<DT>& r, float (&x)[8]) {
+    if constexpr (DT == RT_DT_F32) {
+        x[0] = u2f(r.a.x); x[1] = u2f(r.a.y); x[2] = u2f(r.a.z); x[3] = u2f(r.a.w);
+        x[4] = u2f(r.b.x); x[5] = u2f(r.b.y); x[6] = u2f(r.b.z); x[7] = u2f(r.b.w);
+    } else {
+        const uint32_t w[4] = {r.a.x, r.a.y, r.a.z, r.a.w};
+        if constexpr (DT == RT_DT_BF16) {  // bf16 -> fp32 is the 16 bits moved to the high half
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                x[2 * k] = u2f(w[k] << 16);
+                x[2 * k + 1] = u2f(w[k] & 0xFFFF0000u);
+            }
+        } else {  // IEEE half: v_cvt_f32_f16 is exact
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                x[2 * k] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[k] & 0xFFFFu));
+                x[2 * k + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[k] >> 16));
+            }
+        }
+    }
+}
+
+// Stochastic rounding to bf16: bits(x) + noise16, keep the high half
+// (copy_stochastic_: int32 add, mask 0xFFFF0000).  Two results are packed per
+// word with one byte permute (bytes 2,3 of each sum).
+__device__ __forceinline__ u32x4 sr_pack(const float (&x)[8], u32x4 noise) {
+    const uint32_t nz[4] = {noise.x, noise.y, noise.z, noise.w};
+    uint32_t w[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const uint32_t lo = f2u(x[2 * k]) + (nz[k] & 0xFFFFu);
+        const uint32_t hi = f2u(x[2 * k + 1]) + (nz[k] >> 16);
+        w[k] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);
+    }
+    u32x4 r;
+    r.x = w[0]; r.y = w[1]; r.z = w[2]; r.w = w[3];
+    return r;
+}
+
+// Write-back of one array: bf16 targets are stochastically rounded, fp32
+// targets are stored as they are.
+template <int DT>
+__device__ __forceinline__ void store_out(uint64_t base, uint64_t i, const float (&x)[8], u32x4 noise) {
+    if constexpr (DT == RT_DT_BF16) {
+        stg128(base + i * 2, sr_pack(x, noise));
+    } else {
+        u32x4 a, b;
+        a.x = f2u(x[0]); a.y = f2u(x[1]); a.z = f2u(x[2]); a.w = f2u(x[3]);
+        b.x = f2u(x[4]); b.y = f2u(x[5]); b.z = f2u(x[6]); b.w = f2u(x[7]);
+        stg128(base + i * 4, a);
+        stg128(base + i * 4 + 16, b);
+    }
+}
+
+template <int DT>
+__device__ __forceinline__ void store_out_guarded(uint64_t base, uint64_t i, uint64_t n, const float (&x)[8],
+                                                  u32x4 noise) {
+    if constexpr (DT == RT_DT_BF16) {
+        const u32x4 r = sr_pack(x, noise);
+        const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            if (i + 2 * k < n) stg16(base + (i + 2 * k) * 2, w[k] & 0xFFFFu);
+            if (i + 2 * k + 1 < n) stg16(base + (i + 2 * k + 1) * 2, w[k] >> 16);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if (i + j < n) stg32f(base + (i + j) * 4, x[j]);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// One element of the update in float32, in the rounding sequence of torch's
+// GPU elementwise kernels:
+//   m' = fma(1-b1, g, fl(m*b1))
+//   v' = fma(1-b2, fl(g*g), fl(v*b2))
+//   den = fl(fl(sqrt(v')) * fl(1/bcs)) + eps        (sqrt correctly rounded)
+//   p1 = fl(p * decay)
+//   p' = fma(-step_size, fl(m'/den), p1)            (division correctly rounded)
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void update1(float& p, float g, float& m, float& v, const rt_scalars& s) {
+    const float t = m * s.beta1;
+    const float m1 = __builtin_fmaf(s.one_m_beta1, g, t);
+    const float u = v * s.beta2;
+    const float gg = g * g;
+    const float v1 = __builtin_fmaf(s.one_m_beta2, gg, u);
+    const float sq = __builtin_sqrtf(v1);
+    const float d = sq * s.inv_bcs;
+    const float den = d + s.eps;
+    const float p1 = s.apply_decay ? p * s.decay : p;
+    const float q = m1 / den;
+    p = __builtin_fmaf(s.neg_step_size, q, p1);
+    m = m1;
+    v = v1;
+}
+
+// Per-launch uniform state of the update kernel.
+struct UpdateCtx {
+    rt_scalars s;
+    uint32_t step;
+    uint32_t seed_lo, seed_hi;
+    float coef;
+    bool do_clip;
+    bool do_unscale;
+};
+
+// Noise for the block of 8 elements starting at element i of tensor t.
+template <int PDT, int MDT, int VDT>
+__device__ __forceinline__ void philox_noise3(const DevTensor& t, const UpdateCtx& c, uint64_t i, u32x4& zp,
+                                              u32x4& zm, u32x4& zv) {
+    const uint64_t blk = t.block_base + (i >> 3);
+    const uint32_t b0 = (uint32_t)blk, b1 = (uint32_t)(blk >> 32);
+    if constexpr (PDT == RT_DT_BF16) zp = philox4x32_10(b0, b1, t.tensor_id4 + 0u, c.step, c.seed_lo, c.seed_hi);
+    if constexpr (MDT == RT_DT_BF16) zm = philox4x32_10(b0, b1, t.tensor_id4 + 1u, c.step, c.seed_lo, c.seed_hi);
+    if constexpr (VDT == RT_DT_BF16) zv = philox4x32_10(b0, b1, t.tensor_id4 + 2u, c.step, c.seed_lo, c.seed_hi);
+}
+
+__device__ __forceinline__ void scale_grads(float (&g)[8], const UpdateCtx& c) {
+    if (c.do_unscale) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) g[j] = g[j] * c.s.inv_loss_scale;
+    }
+    if (c.do_clip) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) g[j] = g[j] * c.coef;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Fast path: a chunk that lies wholly inside an aligned tensor.  Every access
+// is a 128-bit global load or store; the loads of vector it+1 are issued
+// before the math of vector it so that memory latency hides behind the VALU
+// work (Philox, sqrt, division).
+// ---------------------------------------------------------------------------
+template <int PDT, int GDT, int MDT, int VDT, int NOISE>
+__device__ __forceinline__ void update_chunk_fast(const DevTensor& t, const UpdateCtx& c, uint64_t chunk_base) {
+    struct In {
+        Raw8<PDT> p;
+        Raw8<GDT> g;
+        Raw8<MDT> m;
+        Raw8<VDT> v;
+        u32x4 zp, zm, zv;
+    };
+    auto fetch = [&](uint64_t i) {
+        In r;
+        r.p = load_raw<PDT>(t.p, i);
+        r.g = load_raw<GDT>(t.g, i);
+        r.m = load_raw<MDT>(t.m, i);
+        r.v = load_raw<VDT>(t.v, i);
+        if constexpr (NOISE == RT_NOISE_EXPLICIT) {
+            if constexpr (PDT == RT_DT_BF16) r.zp = ldg128(t.np + i * 2);
+            if constexpr (MDT == RT_DT_BF16) r.zm = ldg128(t.nm + i * 2);
+            if constexpr (VDT == RT_DT_BF16) r.zv = ldg128(t.nv + i * 2);
+        }
+        return r;
+    };
+    const uint64_t i0 = chunk_base + (uint64_t)threadIdx.x * kVec;
+    In cur = fetch(i0);
+#pragma unroll
+    for (int it = 0; it < kItersPerChunk; ++it) {
+        const uint64_t i = i0 + (uint64_t)it * (kThreads * kVec);
+        In nxt;
+        if (it + 1 < kItersPerChunk) nxt = fetch(i + kThreads * kVec);
+
+        float p[8], g[8], m[8], v[8];
+        decode<PDT>(cur.p, p);
+        decode<GDT>(cur.g, g);
+        decode<MDT>(cur.m, m);
+        decode<VDT>(cur.v, v);
+        u32x4 zp = cur.zp, zm = cur.zm, zv = cur.zv;
+        if constexpr (NOISE == RT_NOISE_PHILOX) philox_noise3<PDT, MDT, VDT>(t, c, i, zp, zm, zv);
+        scale_grads(g, c);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) update1(p[j], g[j], m[j], v[j], c.s);
+        store_out<PDT>(t.p, i, p, zp);
+        store_out<MDT>(t.m, i, m, zm);
+        store_out<VDT>(t.v, i, v, zv);
+        if (it + 1 < kItersPerChunk) cur = nxt;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Generic path: last chunk of a tensor, tensors whose pointers are not
+// 16-byte aligned, debug outputs, gradient centralization.
+// ---------------------------------------------------------------------------
+template <int PDT, int GDT, int MDT, int VDT, int NOISE>
+__device__ __noinline__ void update_chunk_generic(const DevTensor& t, const UpdateCtx& c, uint64_t chunk_base) {
+    const uint64_t n = t.numel;
+    const bool aligned = (t.flags & kFlagAligned) != 0u;
+#pragma unroll 1
+    for (int it = 0; it < kItersPerChunk; ++it) {
+        const uint64_t i = chunk_base + (uint64_t)(it * kThreads + (int)threadIdx.x) * kVec;
+        if (i >= n) break;
+        const bool full = aligned && (i + kVec <= n);
+        Raw8<PDT> rp; Raw8<GDT> rg; Raw8<MDT> rm; Raw8<VDT> rv;
+        u32x4 zp = 0, zm = 0, zv = 0;
+        if (full) {
+            rp = load_raw<PDT>(t.p, i); rg = load_raw<GDT>(t.g, i);
+            rm = load_raw<MDT>(t.m, i); rv = load_raw<VDT>(t.v, i);
+        } else {
+            rp = load_raw_guarded<PDT>(t.p, i, n); rg = load_raw_guarded<GDT>(t.g, i, n);
+            rm = load_raw_guarded<MDT>(t.m, i, n); rv = load_raw_guarded<VDT>(t.v, i, n);
+        }
+        if constexpr (NOISE == RT_NOISE_EXPLICIT) {
+            if constexpr (PDT == RT_DT_BF16)
+                zp = full ? ldg128(t.np + i * 2) : load_raw_guarded<RT_DT_BF16>(t.np, i, n).a;
+            if constexpr (MDT == RT_DT_BF16)
+                zm = full ? ldg128(t.nm + i * 2) : load_raw_guarded<RT_DT_BF16>(t.nm, i, n).a;
+            if constexpr (VDT == RT_DT_BF16)
+                zv = full ? ldg128(t.nv + i * 2) : load_raw_guarded<RT_DT_BF16>(t.nv, i, n).a;
+        } else {
+            philox_noise3<PDT, MDT, VDT>(t, c, i, zp, zm, zv);
+        }
+        float p[8], g[8], m[8], v[8];
+        decode<PDT>(rp, p); decode<GDT>(rg, g); decode<MDT>(rm, m); decode<VDT>(rv, v);
+        scale_grads(g, c);
+        if (t.row_mean != 0) {
+            // grad.sub_(mean.mul_(c)): the product is rounded, then subtracted.
+            const uint64_t e0 = (t.block_base << 3) + i;
+#pragma unroll 1
+            for (int j = 0; j < 8; ++j) {
+                if (i + j >= n) break;
+                const uint64_t row = (e0 + j) / t.row_len;
+                const float mc = ldg32f(t.row_mean + row * 4) * c.s.centralization;
+                g[j] = g[j] - mc;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) update1(p[j], g[j], m[j], v[j], c.s);
+
+        if (t.dp != 0) store_out_guarded<RT_DT_F32>(t.dp, i, n, p, zp);
+        if (t.dm != 0) store_out_guarded<RT_DT_F32>(t.dm, i, n, m, zm);
+        if (t.dv != 0) store_out_guarded<RT_DT_F32>(t.dv, i, n, v, zv);
+        if (full) {
+            store_out<PDT>(t.p, i, p, zp);
+            store_out<MDT>(t.m, i, m, zm);
+            store_out<VDT>(t.v, i, v, zv);
+        } else {
+            store_out_guarded<PDT>(t.p, i, n, p, zp);
+            store_out_guarded<MDT>(t.m, i, n, m, zm);
+            store_out_guarded<VDT>(t.v, i, n, v, zv);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Multi-tensor update: one workgroup per ChunkRef.
+// ---------------------------------------------------------------------------
+template <int PDT, int GDT, int MDT, int VDT, int NOISE>
+__global__ __launch_bounds__(kThreads) void sr_adamw_multi_kernel(
+    const DevTensor* __restrict__ tensors, const ChunkRef* __restrict__ chunks,
+    const DevScalars* __restrict__ sets, uint32_t seed_lo, uint32_t seed_hi,
+    const float* __restrict__ clip_coef, const uint32_t* __restrict__ skip) {
+    if (skip != nullptr && *skip != 0u) return;
+
+    const ChunkRef cr = chunks[blockIdx.x];
+    const DevTensor& t = tensors[cr.tensor];
+    const DevScalars& set = sets[t.set_idx];
+    UpdateCtx c;
+    c.s = set.s;
+    c.step = set.step;
+    c.seed_lo = seed_lo;
+    c.seed_hi = seed_hi;
+    c.do_clip = clip_coef != nullptr;
+    c.coef = c.do_clip ? *clip_coef : 1.0f;
+    c.do_unscale = c.s.inv_loss_scale != 1.0f;
+
+    const uint64_t chunk_base = (uint64_t)cr.chunk * kChunkElems;
+    const bool fast = (t.flags & kFlagAligned) != 0u && chunk_base + kChunkElems <= t.numel &&
+                      (t.dp | t.dm | t.dv | t.row_mean) == 0;
+    if (fast) update_chunk_fast<PDT, GDT, MDT, VDT, NOISE>(t, c, chunk_base);
+    else update_chunk_generic<PDT, GDT, MDT, VDT, NOISE>(t, c, chunk_base);
+}
+
+// ---------------------------------------------------------------------------
+// copy_stochastic_ on its own: fp32 -> bf16.  Philox counter word 2 is 3
+// ("which" values 0..2 belong to the step), word 3 is 0.
+// ---------------------------------------------------------------------------
+template <int NOISE>
+__global__ __launch_bounds__(kThreads) void sr_copy_kernel(uint64_t target, uint64_t source, uint64_t n,
+                                                           uint64_t noise, uint32_t seed_lo, uint32_t seed_hi,
+                                                           int aligned) {
+    const uint64_t stride = (uint64_t)gridDim.x * kThreads * kVec;
+    for (uint64_t i = ((uint64_t)blockIdx.x * kThreads + threadIdx.x) * kVec; i < n; i += stride) {
+        const bool full = aligned && (i + kVec <= n);
+        const Raw8<RT_DT_F32> r = full ? load_raw<RT_DT_F32>(source, i) : load_raw_guarded<RT_DT_F32>(source, i, n);
+        float x[8];
+        decode<RT_DT_F32>(r, x);
+        u32x4 z;
+        if constexpr (NOISE == RT_NOISE_EXPLICIT) {
+            z = full ? ldg128(noise + i * 2) : load_raw_guarded<RT_DT_BF16>(noise, i, n).a;
+        } else {
+            const uint64_t blk = i >> 3;
+            z = philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), 3u, 0u, seed_lo, seed_hi);
+        }
+        if (full) store_out<RT_DT_BF16>(target, i, x, z);
+        else store_out_guarded<RT_DT_BF16>(target, i, n, x, z);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Wavefront / workgroup sum in a fixed order (deterministic run to run).
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) x = x + __shfl_xor(x, off, 64);
+    return x;
+}
+
+__device__ __forceinline__ float block_sum(float x, float* lds) {
+    x = wave_sum(x);
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) lds[wave] = x;
+    __syncthreads();
+    float r = 0.0f;
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 0; w < kThreads / 64; ++w) r = r + lds[w];
+    }
+    __syncthreads();
+    return r;  // valid in thread 0
+}
+
+// Sum of squares of one chunk of one gradient tensor (per-lane partial).
+template <int GDT>
+__device__ __forceinline__ float chunk_sumsq(const DevTensor& t, uint32_t chunk, float inv_loss_scale) {
+    const uint64_t n = t.numel;
+    const uint64_t chunk_base = (uint64_t)chunk * kChunkElems;
+    const bool aligned = (t.g & 15u) == 0;
+    float acc = 0.0f;
+#pragma unroll 1
+    for (int it = 0; it < kItersPerChunk; ++it) {
+        const uint64_t i = chunk_base + (uint64_t)(it * kThreads + (int)threadIdx.x) * kVec;
+        if (i >= n) break;
+        const bool full = aligned && (i + kVec <= n);
+        const Raw8<GDT> r = full ? load_raw<GDT>(t.g, i) : load_raw_guarded<GDT>(t.g, i, n);
+        float g[8];
+        decode<GDT>(r, g);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float x = g[j] * inv_loss_scale;
+            acc = __builtin_fmaf(x, x, acc);
+        }
+    }
+    return acc;
+}
+
+// Pass 1 of the global grad norm: workgroup b accumulates the chunks
+// b, b + gridDim.x, ... and writes one partial sum of squares.
+__global__ __launch_bounds__(kThreads) void grad_sumsq_kernel(const DevTensor* __restrict__ tensors,
+                                                              const ChunkRef* __restrict__ chunks,
+                                                              uint32_t n_chunks, const uint8_t* __restrict__ gdt,
+                                                              float inv_loss_scale, double* __restrict__ partials) {
+    __shared__ float lds[kThreads / 64];
+    double total = 0.0;
+    for (uint32_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+        const ChunkRef cr = chunks[c];
+        const DevTensor& t = tensors[cr.tensor];
+        const int dt = gdt[cr.tensor];
+        float acc;
+        if (dt == RT_DT_BF16) acc = chunk_sumsq<RT_DT_BF16>(t, cr.chunk, inv_loss_scale);
+        else if (dt == RT_DT_F32) acc = chunk_sumsq<RT_DT_F32>(t, cr.chunk, inv_loss_scale);
+        else acc = chunk_sumsq<RT_DT_F16>(t, cr.chunk, inv_loss_scale);
+        const float bs = block_sum(acc, lds);
+        total += (double)bs;  // meaningful in thread 0 only
+    }
+    if (threadIdx.x == 0) partials[blockIdx.x] = total;
+}
+
+// Pass 2: one workgroup folds the partials in index order and derives the
+// clip coefficient with torch.nn.utils.clip_grad_norm_'s formula.
+__global__ __launch_bounds__(kThreads) void grad_norm_finish_kernel(const double* __restrict__ partials,
+                                                                    uint32_t n_partials, float max_norm,
+                                                                    float* __restrict__ out) {
+    __shared__ double lds[kThreads];
+    double acc = 0.0;
+    for (uint32_t i = threadIdx.x; i < n_partials; i += kThreads) acc += partials[i];
+    lds[threadIdx.x] = acc;
+    __syncthreads();
+    for (int w = kThreads / 2; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) lds[threadIdx.x] += lds[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        const float total = (float)__builtin_sqrt(lds[0]);
+        const bool finite = (f2u(total) & 0x7F800000u) != 0x7F800000u;
+        const float c = max_norm / (total + 1e-6f);
+        out[0] = total;
+        // a non-finite norm must never scale anything: the skip flag stops the update
+        out[1] = (finite && c < 1.0f) ? c : 1.0f;
+        ((uint32_t*)out)[2] = finite ? 0u : 1u;
+    }
+}
+
+// Row means for centralization: one workgroup per row.
+template <int GDT>
+__global__ __launch_bounds__(kThreads) void row_mean_kernel(uint64_t g, uint64_t row_len, float inv_loss_scale,
+                                                            float* __restrict__ out) {
+    __shared__ float lds[kThreads / 64];
+    const uint64_t row = blockIdx.x;
+    const uint64_t base = row * row_len;
+    const bool aligned = (g & 15u) == 0 && (row_len % kVec) == 0;
+    float acc = 0.0f;
+    for (uint64_t c = (uint64_t)threadIdx.x * kVec; c < row_len; c += (uint64_t)kThreads * kVec) {
+        const bool full = aligned && (c + kVec <= row_len);
+        const Raw8<GDT> r = full ? load_raw<GDT>(g, base + c) : load_raw_guarded<GDT>(g, base + c, base + row_len);
+        float x[8];
+        decode<GDT>(r, x);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc = acc + x[j] * inv_loss_scale;
+    }
+    const float sum = block_sum(acc, lds);
+    if (threadIdx.x == 0) out[row] = sum / (float)row_len;
+}
+
+}  // namespace rt

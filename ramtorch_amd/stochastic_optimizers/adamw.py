@@ -1,0 +1,252 @@
+"""``ramtorch.AdamW`` on MI355X: the same optimizer interface as the reference's
+``ramtorch/stochastic_optimizers/adamw.py`` (constructor arguments, ``param_groups``,
+``state[p] = {"step", "ema", "ema_squared"}``, ``step()``, inherited
+``state_dict`` / ``load_state_dict``), with the per-tensor loop of torch ops
+replaced by one fused HIP launch over all tensors (GPU-resident tensors) or by
+a chunked H2D / update / D2H pipeline (tensors held in host memory).
+
+There is no CPU or eager fallback: ``step()`` needs the HIP library and a GPU.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+from torch.optim import Optimizer
+
+from .. import _native as N
+from .. import functional as F
+
+_handles: Dict[int, N.Handle] = {}
+
+
+def _handle(device_index: int) -> N.Handle:
+    h = _handles.get(device_index)
+    if h is None:
+        h = _handles[device_index] = N.Handle(device_index)
+    return h
+
+
+def _compute_device_index(p: torch.Tensor) -> int:
+    # adamw.py:152-157: CPU params are computed on the current GPU
+    if p.is_cuda:
+        return p.device.index if p.device.index is not None else torch.cuda.current_device()
+    return torch.cuda.current_device()
+
+
+def copy_stochastic_(target: torch.Tensor, source: torch.Tensor, seed=0, *, noise: Optional[torch.Tensor] = None):
+    """Stochastically round fp32 ``source`` into bf16 ``target`` (adamw.py:6-30):
+    add 16 random bits below the bf16 mantissa, keep the high half.
+
+    The reference draws the bits with ``torch.randint`` from a generator seeded
+    with ``seed``; here they come from Philox4x32-10 keyed by ``seed`` (or from
+    ``noise``, an int16 tensor, for reproducible tests).  Both tensors must be
+    contiguous GPU tensors; a CPU ``target`` is filled through a GPU temporary.
+    """
+    if source.dtype != torch.float32 or target.dtype != torch.bfloat16:
+        raise TypeError("copy_stochastic_ rounds float32 -> bfloat16")
+    if source.numel() != target.numel():
+        raise ValueError("target and source sizes differ")
+    with torch.no_grad():
+        if not source.is_cuda:
+            raise RuntimeError("copy_stochastic_ needs a GPU source tensor (no CPU implementation)")
+        N.lib()
+        src = source.contiguous()
+        dst = target if (target.is_cuda and target.is_contiguous()) else torch.empty(
+            target.shape, dtype=torch.bfloat16, device=source.device)
+        nz = None
+        if noise is not None:
+            if noise.dtype not in (torch.int16, torch.uint16) or noise.numel() != source.numel():
+                raise ValueError("noise must be an int16 tensor of source's size")
+            nz = noise.to(source.device).contiguous()
+        with torch.cuda.device(source.device):
+            stream = torch.cuda.current_stream().cuda_stream
+            N.sr_copy(dst.data_ptr(), src.data_ptr(), src.numel(), None if nz is None else nz.data_ptr(),
+                      int(seed) & (2 ** 64 - 1), stream)
+        if dst is not target:
+            target.copy_(dst)  # bf16 -> bf16, exact
+    return target
+
+
+class AdamW(Optimizer):
+    r"""AdamW with bf16 stochastic rounding of parameters and states.
+
+    Arguments (same meaning and defaults as the reference, adamw.py:57-69):
+        params: iterable of parameters or of param-group dicts (for instance one
+            rank's list from ``create_zero_param_groups``; empty groups are fine).
+        lr (float, default 1e-3), betas (default (0.9, 0.999)), eps (default 1e-8),
+        weight_decay (default 1e-2): decoupled decay, applied as
+            ``p *= 1 - (lr / bias_correction) * weight_decay`` (adamw.py:188,198).
+        centralization (default 0): subtract ``c *`` row mean from each gradient.
+        chunk_size (default 64): kept for interface compatibility; the fused step
+            has no per-tensor synchronisation to space out.
+        dtype (default bfloat16): dtype of ``ema`` / ``ema_squared``.
+        storage_device (default "cpu"): where the states live; "cpu" states are pinned.
+
+    Keyword-only additions (not in the reference):
+        seed: Philox key of the rounding noise.
+        stream_chunk_bytes: bytes of bf16 per staged chunk of the host-resident path.
+        loss_scale: gradients are divided by this inside the kernel.
+        max_grad_norm: global L2 clip computed on the GPU before the update.
+    """
+
+    def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=1e-2, centralization=0,
+                 chunk_size=64, dtype=torch.bfloat16, storage_device="cpu", *, seed: int = 0,
+                 stream_chunk_bytes: int = 256 << 20, loss_scale: float = 1.0,
+                 max_grad_norm: Optional[float] = None):
+        defaults = dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay, centralization=centralization)
+        super().__init__(params, defaults)
+        self.chunk_size = chunk_size
+        self.optim_state_dtype = dtype
+        self.optim_state_device = storage_device
+        self.seed = int(seed)
+        self.stream_chunk_bytes = int(stream_chunk_bytes)
+        self.loss_scale = float(loss_scale)
+        self.max_grad_norm = max_grad_norm
+        self.last_grad_norm: Optional[torch.Tensor] = None  # [norm, clip_coef, found_inf bits, -] on the GPU
+        # eager state allocation, as adamw.py:84-104
+        for group in self.param_groups:
+            for p in group["params"]:
+                if not self.state[p]:
+                    self._init_state(p)
+
+    # -- state ---------------------------------------------------------------------
+    def _new_state_tensor(self, p: torch.Tensor) -> torch.Tensor:
+        t = torch.zeros_like(p.data, dtype=self.optim_state_dtype, device=self.optim_state_device,
+                             memory_format=torch.contiguous_format)
+        if self.optim_state_device == "cpu" and torch.cuda.is_available():
+            # adamw.py:91-97 pins unconditionally; without a GPU there is nothing to pin for
+            t = t.pin_memory()
+        return t
+
+    def _init_state(self, p: torch.Tensor) -> None:
+        state = self.state[p]
+        state["step"] = 0
+        state["ema"] = self._new_state_tensor(p)
+        state["ema_squared"] = self._new_state_tensor(p)
+
+    def _tensor_ids(self) -> Dict[int, int]:
+        ids: Dict[int, int] = {}
+        k = 0
+        for group in self.param_groups:
+            for p in group["params"]:
+                ids[id(p)] = k
+                k += 1
+        return ids
+
+    # -- step ----------------------------------------------------------------------
+    def step(self, closure=None, *, noise=None, debug_out=None):
+        """One optimizer step (adamw.py:106-234).
+
+        ``noise``: optional ``{param: (noise_p, noise_m, noise_v)}`` of int16 GPU
+        tensors -- the explicit-noise test mode (every stepped bf16 array needs one).
+        ``debug_out``: optional ``{param: (p32, m32, v32)}`` fp32 GPU tensors that
+        receive the values before rounding.
+        """
+        loss = None
+        if closure is not None:
+            loss = closure()
+
+        N.lib()  # fail loudly before touching any state if the extension is missing
+        if not torch.cuda.is_available():
+            raise RuntimeError("ramtorch_amd.AdamW.step needs a GPU: the update runs only as HIP kernels")
+
+        ids = self._tensor_ids()
+        scalars: List[N.RtScalars] = []
+        scalar_key: Dict[tuple, int] = {}
+        resident: Dict[int, List[F.Entry]] = {}
+        streamed: Dict[int, List[F.Entry]] = {}
+        writeback = []  # (destination, contiguous temporary) pairs for non-contiguous p / states
+        inv_loss_scale = 1.0 / self.loss_scale if self.loss_scale != 1.0 else 1.0
+
+        with torch.no_grad():
+            for gi, group in enumerate(self.param_groups):
+                beta1, beta2 = group["betas"]
+                for p in group["params"]:
+                    if p.grad is None:
+                        continue  # adamw.py:114: skipped, and its step count does not advance
+                    grad = p.grad
+                    if grad.is_sparse:
+                        raise RuntimeError("AdamW does not support sparse gradients")  # adamw.py:118-119
+                    state = self.state[p]
+                    if not state:
+                        self._init_state(p)  # adamw.py:125-148
+                    dev = _compute_device_index(p)
+                    state["step"] += 1  # adamw.py:177
+                    step = state["step"]
+                    key = (gi, step, group["lr"], beta1, beta2, group["eps"], group["weight_decay"],
+                           group["centralization"])
+                    si = scalar_key.get(key)
+                    if si is None:
+                        si = scalar_key[key] = len(scalars)
+                        scalars.append(F.make_scalars(group["lr"], (beta1, beta2), group["eps"],
+                                                      group["weight_decay"], step,
+                                                      centralization=group["centralization"],
+                                                      inv_loss_scale=inv_loss_scale))
+                    keep = []
+                    pt, mt, vt = p.data, state["ema"], state["ema_squared"]
+                    arrays = []
+                    for t in (pt, mt, vt):
+                        if t.is_cuda and t.device.index != dev:
+                            raise RuntimeError("param and optimizer states live on different GPUs")
+                        if not t.is_contiguous():
+                            c = t.contiguous()
+                            writeback.append((t, c))
+                            t = c
+                        arrays.append(t)
+                    g = grad.detach()
+                    if g.is_cuda and g.device.index != dev:
+                        g = g.to(f"cuda:{dev}")
+                    if not g.is_contiguous():
+                        g = g.contiguous()
+                    if g.dtype not in (torch.bfloat16, torch.float32, torch.float16):
+                        g = g.to(torch.float32)  # adamw.py:167 upcasts every gradient to fp32
+                    e = F.Entry(p=arrays[0], g=g, m=arrays[1], v=arrays[2], step=step, scalars_idx=si,
+                                tensor_id=ids[id(p)], keep=keep)
+                    if group["centralization"] != 0:
+                        if self.max_grad_norm is not None:
+                            raise NotImplementedError("centralization together with max_grad_norm")
+                        if not g.is_cuda:
+                            g = g.to(f"cuda:{dev}", non_blocking=True)
+                            e.g = g
+                        # adamw.py:179-184: mean over every dim but the first (all dims for 0-d / 1-d)
+                        rows = g.shape[0] if g.dim() >= 2 else 1
+                        row_len = g.numel() // rows if rows else 0
+                        if g.numel():
+                            with torch.cuda.device(dev):
+                                e.row_mean = F.row_means(_handle(dev), g, rows, row_len, inv_loss_scale)
+                            e.row_len = row_len
+                    if noise is not None and p in noise:
+                        e.noise = tuple(noise[p])
+                    if debug_out is not None and p in debug_out:
+                        e.dbg = tuple(debug_out[p])
+                    on_gpu = e.p.is_cuda and e.g.is_cuda and e.m.is_cuda and e.v.is_cuda
+                    (resident if on_gpu else streamed).setdefault(dev, []).append(e)
+
+            explicit = noise is not None
+            for dev in sorted(set(resident) | set(streamed)):
+                h = _handle(dev)
+                with torch.cuda.device(dev):
+                    res, stm = resident.get(dev, []), streamed.get(dev, [])
+                    clip = skip = None
+                    if self.max_grad_norm is not None:
+                        if stm:
+                            raise NotImplementedError("max_grad_norm with host-resident params or states")
+                        grads = [e.g for e in res + stm]
+                        for i, g in enumerate(grads):
+                            if not g.is_cuda:
+                                grads[i] = g.to(f"cuda:{dev}", non_blocking=True)
+                        for e, g in zip(res + stm, grads):
+                            e.g = g
+                        out = F.grad_norm(h, grads, inv_loss_scale=inv_loss_scale, max_norm=self.max_grad_norm)
+                        self.last_grad_norm = out
+                        clip, skip = out[1:2], out[2:3]
+                    F.step_resident(h, res, scalars, seed=self.seed, explicit_noise=explicit, clip_coef=clip,
+                                    skip=skip)
+                    if stm:
+                        chunk_elems = max(8, (self.stream_chunk_bytes // 2) // 8 * 8)
+                        F.step_streamed(h, stm, scalars, seed=self.seed, explicit_noise=explicit,
+                                        chunk_elems=chunk_elems)
+            for dst, tmp in writeback:
+                dst.copy_(tmp)
+        return loss
