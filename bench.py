@@ -1,0 +1,325 @@
+#!/usr/bin/env python3
+"""Benchmark of the SR-AdamW step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama8b]
+
+A "step" is one ``AdamW.step()`` over the whole synthetic parameter set, with
+params, grads and both states already resident in HBM (or, for the streamed
+workload, params/states in pinned host memory).  Prints ONE JSON line:
+
+  value      elements updated per second over the K timed steps (wall clock
+             around the steps, device synchronised on both sides)
+  roofline   algorithmic HBM bytes per launch / mean kernel time of the update
+             kernel, the kernel time taken with HIP events on the launch stream
+             inside the library; peak = 8 TB/s
+  cpu_baseline  the same ATen op sequence the reference issues
+             (ramtorch/stochastic_optimizers/adamw.py:160-222), on CPU tensors
+             with all host threads, on a bounded sample; plus the scalar C
+             oracle on one thread
+
+Workloads (synthetic, value distributions param~N(0,0.02), grad~N(0,1e-3),
+ema~N(0,1e-4), ema_squared=N(0,1e-3)^2, stored bf16):
+  llama8b   Llama-3-8B-shaped set, 290 tensors, 8 030 257 152 elements, all bf16,
+            Philox seed 1234, first timed step is step 100            [default]
+  cfg0      one 4096x4096 weight, explicit int16 noise, step 10
+  small     20 000 small tensors (length log-uniform in [1,4096]) + 64 x 1024x1024
+  mixed     Llama-3-8B shapes; bf16 p and ema, fp32 ema_squared, fp32 grads scaled
+            by 1024 and unscaled in-kernel, global-norm clip to 1.0
+  streamed  Llama-3-8B shapes with p/ema/ema_squared in pinned host memory,
+            bf16 grads on the GPU, 256 MB chunks (--stream-gb bounds the host set)
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
+METRIC = "SR-AdamW step: params/sec + achieved HBM GB/s (% of peak), 8B bf16 set, 1 GPU"
+
+
+# ---- workload shapes -------------------------------------------------------------------------
+def llama3_8b_shapes(layers: int = 32):
+    """embed and lm_head 128256x4096; per layer q/o 4096x4096, k/v 1024x4096,
+    gate/up 14336x4096, down 4096x14336, two RMSNorm vectors of 4096."""
+    shapes = [(128256, 4096)]
+    for _ in range(layers):
+        shapes += [(4096, 4096), (1024, 4096), (1024, 4096), (4096, 4096),      # q k v o
+                   (14336, 4096), (14336, 4096), (4096, 14336), (4096,), (4096,)]
+    shapes.append((128256, 4096))
+    return shapes
+
+
+def small_tensor_shapes(seed: int = 1234, count: int = 20_000, big: int = 64):
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    lens = np.floor(np.exp(rng.uniform(0.0, math.log(4096.0), count))).astype(np.int64).clip(1, 4096)
+    return [(int(n),) for n in lens] + [(1024, 1024)] * big
+
+
+def numel(shape):
+    n = 1
+    for s in shape:
+        n *= s
+    return n
+
+
+def fill_tensor(shape, kind: str, seed: int, dtype, device):
+    """Synthetic values of one array, drawn in fp32 on `device` and stored as `dtype`."""
+    import torch
+    gen = torch.Generator(device=device).manual_seed(seed)
+    n = numel(shape)
+    out = torch.empty(n, dtype=dtype, device=device)
+    step = 1 << 28  # bound the fp32 temporary
+    for lo in range(0, n, step):
+        k = min(step, n - lo)
+        x = torch.randn(k, device=device, generator=gen)
+        if kind == "p":
+            x.mul_(0.02)
+        elif kind == "g":
+            x.mul_(1e-3)
+        elif kind == "m":
+            x.mul_(1e-4)
+        else:
+            x.mul_(1e-3).square_()
+        out[lo:lo + k] = x
+    return out.view(shape)
+
+
+def cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+# ---- CPU baseline ----------------------------------------------------------------------------
+def cpu_baseline(sample_elems: int = 4096 * 4096):
+    """The reference's op sequence on CPU tensors (its CPU path cannot run
+    without a GPU, so this restatement is what is timed), all host threads,
+    including the three randint draws the reference pays for.  Bounded sample:
+    one 4096x4096 bf16 weight, best of 3 after a warm-up."""
+    import numpy as np
+    import torch
+    import oracle
+    from oracle import torch_ops
+
+    n = sample_elems
+    shape = (4096, n // 4096) if n % 4096 == 0 else (n,)
+    P = fill_tensor(shape, "p", 1, torch.bfloat16, "cpu")
+    G = fill_tensor(shape, "g", 2, torch.bfloat16, "cpu")
+    M = fill_tensor(shape, "m", 3, torch.bfloat16, "cpu")
+    V = fill_tensor(shape, "v", 4, torch.bfloat16, "cpu")
+    best = float("inf")
+    for it in range(4):
+        t0 = time.perf_counter()
+        torch_ops.reference_step_ops(P, G, M, V, step=10 + it, noise=None, **HP)
+        dt = time.perf_counter() - t0
+        if it:
+            best = min(best, dt)
+    threads = torch.get_num_threads()
+
+    # scalar C restatement, one thread, explicit noise (no RNG cost)
+    k = 1 << 22
+    p, g, m, v = oracle.synth_inputs(k, 1)
+    noise = oracle.synth_noise(k, 1)
+    sc = oracle.scalars_from_hparams(step=10, **HP)
+    t0 = time.perf_counter()
+    oracle.step_tensor(p, g, m, v, sc, noise=noise)
+    c_dt = time.perf_counter() - t0
+    return {
+        "value": n / best, "unit": "elements/s", "cores": threads, "kind": "port",
+        "sample": f"torch-op restatement of adamw.py:160-222 on CPU tensors, one {shape[0]}x{shape[-1]} bf16 weight, "
+                  f"best of 3, {threads} threads, {cpu_model()}",
+        "ms_per_sample": best * 1e3,
+        "c_oracle_1thread_elements_per_s": k / c_dt,
+    }
+
+
+# ---- GPU workloads ----------------------------------------------------------------------------
+def build_resident(shapes, *, g_dtype, v_dtype, device, seed=1234):
+    import torch
+    params, grads = [], []
+    for i, shp in enumerate(shapes):
+        p = torch.nn.Parameter(fill_tensor(shp, "p", seed + 4 * i, torch.bfloat16, device), requires_grad=False)
+        g = fill_tensor(shp, "g", seed + 4 * i + 1, torch.float32 if g_dtype == torch.float32 else torch.bfloat16,
+                        device)
+        if g_dtype == torch.float32:
+            g.mul_(1024.0)
+        params.append(p)
+        grads.append(g)
+    return params, grads
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="llama8b", choices=["llama8b", "cfg0", "small", "mixed", "streamed"])
+    ap.add_argument("--layers", type=int, default=32, help="transformer layers of the Llama-shaped set")
+    ap.add_argument("--stream-gb", type=float, default=48.2, help="upper bound on pinned host bytes (streamed)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; the step needs no exchange between GPUs and a multi-GPU "
+              "figure is not part of it (it would shard by tensor, as ZeRO-1 does). Use --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+    import ramtorch_amd
+    from ramtorch_amd.stochastic_optimizers import adamw as adamw_mod
+
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X", file=sys.stderr)
+        return 1
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    wl = args.workload
+    first_step = 100
+    noise = None
+    opt_kw = dict(storage_device="cuda", seed=1234)
+    bytes_per_elem = 14
+    dtype_label = "bf16 storage, f32 arithmetic"
+    if wl == "llama8b":
+        shapes = llama3_8b_shapes(args.layers)
+        params, grads = build_resident(shapes, g_dtype=torch.bfloat16, v_dtype=torch.bfloat16, device=dev)
+        state_dtype = torch.bfloat16
+    elif wl == "cfg0":
+        shapes = [(4096, 4096)]
+        params, grads = build_resident(shapes, g_dtype=torch.bfloat16, v_dtype=torch.bfloat16, device=dev)
+        state_dtype = torch.bfloat16
+        first_step = 10
+        bytes_per_elem = 20
+    elif wl == "small":
+        shapes = small_tensor_shapes()
+        params, grads = build_resident(shapes, g_dtype=torch.bfloat16, v_dtype=torch.bfloat16, device=dev)
+        state_dtype = torch.bfloat16
+    elif wl == "mixed":
+        shapes = llama3_8b_shapes(args.layers)
+        params, grads = build_resident(shapes, g_dtype=torch.float32, v_dtype=torch.float32, device=dev)
+        state_dtype = torch.bfloat16
+        opt_kw.update(loss_scale=1024.0, max_grad_norm=1.0)
+        bytes_per_elem = 24
+    else:  # streamed
+        shapes = llama3_8b_shapes(args.layers)
+        budget = int(args.stream_gb * 1e9)
+        kept, used = [], 0
+        for shp in shapes:
+            if used + 6 * numel(shp) > budget:
+                break
+            kept.append(shp)
+            used += 6 * numel(shp)
+        shapes = kept
+        params, grads = [], []
+        for i, shp in enumerate(shapes):
+            p = fill_tensor(shp, "p", 1234 + 4 * i, torch.bfloat16, dev).cpu().pin_memory()
+            params.append(torch.nn.Parameter(p, requires_grad=False))
+            grads.append(fill_tensor(shp, "g", 1234 + 4 * i + 1, torch.bfloat16, dev))
+        state_dtype = torch.bfloat16
+        opt_kw = dict(storage_device="cpu", seed=1234, stream_chunk_bytes=256 << 20)
+        bytes_per_elem = 12
+
+    total = sum(numel(s) for s in shapes)
+    opt = ramtorch_amd.AdamW(params, dtype=state_dtype, **HP, **opt_kw)
+    for i, p in enumerate(params):
+        st = opt.state[p]
+        st["step"] = first_step - 1 - args.warmup
+        if wl != "streamed":
+            st["ema"] = fill_tensor(p.shape, "m", 1234 + 4 * i + 2, torch.bfloat16, dev)
+            vdt = torch.float32 if wl == "mixed" else torch.bfloat16
+            st["ema_squared"] = fill_tensor(p.shape, "v", 1234 + 4 * i + 3, vdt, dev)
+        else:
+            st["ema"].copy_(fill_tensor(p.shape, "m", 1234 + 4 * i + 2, torch.bfloat16, dev))
+            st["ema_squared"].copy_(fill_tensor(p.shape, "v", 1234 + 4 * i + 3, torch.bfloat16, dev))
+    if wl == "cfg0":
+        noise = {params[0]: tuple(torch.randint(-32768, 32768, (4096, 4096), dtype=torch.int16, device=dev,
+                                                generator=torch.Generator(dev).manual_seed(1234 + k))
+                                  for k in (1, 2, 3))}
+    gmap = dict(zip(params, grads))
+    torch.cuda.synchronize()
+
+    handle = adamw_mod._handle(0)
+    for _ in range(args.warmup):
+        opt.step(noise=noise, grads=gmap)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        opt.step(noise=noise, grads=gmap)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+
+    # kernel time of the update launch, HIP events on the launch stream (separate pass so
+    # that reading the events does not serialise the timed region above)
+    roofline = None
+    stream_info = None
+    if wl != "streamed":
+        handle.set_timing(True)
+        ks = []
+        for _ in range(min(args.steps, 10)):
+            opt.step(noise=noise, grads=gmap)
+            ks.append(handle.last_kernel_ms())
+        handle.set_timing(False)
+        k_ms = sum(ks) / len(ks)
+        # the update launch moves 14 (20 with explicit noise; 20 for the mixed layout, whose
+        # norm pass is a separate launch of 4 B/elem) bytes per element
+        upd_bytes = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 20}[wl] * total
+        achieved = upd_bytes / (k_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                    "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "sr_adamw_multi_kernel",
+                    "kernel_ms": k_ms, "algorithmic_bytes_per_launch": upd_bytes}
+    else:
+        st = handle.streamed_stats()
+        stream_info = {"h2d_GBps": st["bytes_h2d"] / st["seconds"] / 1e9, "d2h_GBps": st["bytes_d2h"] / st["seconds"] / 1e9,
+                       "seconds_last_call": st["seconds"], "host_bytes": 6 * total}
+        # same-run pinned-copy peaks with the same chunk size
+        chunk = 256 << 20
+        hbuf = torch.empty(chunk, dtype=torch.uint8).pin_memory()
+        dbuf = torch.empty(chunk, dtype=torch.uint8, device=dev)
+        for name, (dst, src) in (("h2d", (dbuf, hbuf)), ("d2h", (hbuf, dbuf))):
+            dst.copy_(src, non_blocking=True)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for _ in range(8):
+                dst.copy_(src, non_blocking=True)
+            torch.cuda.synchronize()
+            stream_info[f"pinned_{name}_peak_GBps"] = 8 * chunk / (time.perf_counter() - t1) / 1e9
+        stream_info["h2d_frac_of_peak"] = stream_info["h2d_GBps"] / stream_info["pinned_h2d_peak_GBps"]
+        roofline = {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": None,
+                    "traffic": None, "note": "host-link bound; see host_link"}
+
+    out = {
+        "metric": METRIC, "value": total / (ms_per_step * 1e-3), "unit": "elements/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": dtype_label, "data": "synthetic",
+        "config": {"workload": wl, "tensors": len(shapes), "elements": total, "bytes_per_element": bytes_per_elem,
+                   "first_timed_step": first_step, "noise": "explicit int16" if noise else "philox seed 1234",
+                   "hparams": {"lr": HP["lr"], "betas": list(HP["betas"]), "eps": HP["eps"],
+                               "weight_decay": HP["weight_decay"]}},
+        "achieved_GBps_wall": bytes_per_elem * total / (ms_per_step * 1e-3) / 1e9,
+        "roofline": roofline,
+    }
+    if stream_info:
+        out["host_link"] = stream_info
+    if not args.no_cpu_baseline:
+        del params, grads, opt, gmap
+        torch.cuda.empty_cache()
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -53,7 +53,7 @@ typedef struct rt_scalars {
     float one_m_beta1;    /* float32(1 - beta1)                  adamw.py:190 */
     float beta2;          /* float32(beta2)                      adamw.py:191 */
     float one_m_beta2;    /* float32(1 - beta2)                  adamw.py:191 */
-    float inv_bcs;        /* 1.0f / float32(sqrt(1 - beta2^t))   adamw.py:187,193 */
+    float inv_bcs;        /* float32(1.0 / sqrt(1 - beta2^t))    adamw.py:187,193 */
     float eps;            /* float32(eps)                        adamw.py:194 */
     float decay;          /* float32(1 - (lr/bc) * wd)           adamw.py:188,198 */
     float neg_step_size;  /* float32(-(lr/bc))                   adamw.py:188,200 */

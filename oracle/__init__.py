@@ -116,7 +116,9 @@ def scalars_from_hparams(lr, betas, eps, weight_decay, step, inv_loss_scale=1.0,
         beta2=np.float32(beta2),
         one_m_beta2=np.float32(1 - beta2),
         bcs=bcs32,
-        inv_bcs=np.float32(1.0) / bcs32,
+        # torch's GPU `tensor / python_float` multiplies by the reciprocal taken in double and
+        # then rounded to float32 (pinned by tests/golden/torch_gpu_step.npz, case step1)
+        inv_bcs=np.float32(1.0 / bias_correction_sqrt),
         eps=np.float32(eps),
         decay=np.float32(1 - step_size * weight_decay),
         neg_step_size=np.float32(-step_size),

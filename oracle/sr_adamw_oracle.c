@@ -47,7 +47,7 @@ typedef struct orc_scalars {
     float beta2;          /* float32(beta2)                         adamw.py:191 */
     float one_m_beta2;    /* float32(1 - beta2)                     adamw.py:191 */
     float bcs;            /* float32((1 - beta2**step) ** 0.5)      adamw.py:187 */
-    float inv_bcs;        /* 1.0f / bcs evaluated in float32        adamw.py:193 */
+    float inv_bcs;        /* float32(1.0 / bcs), reciprocal in double  adamw.py:193 */
     float eps;            /* float32(eps)                           adamw.py:194 */
     float decay;          /* float32(1 - (lr/bc) * wd)              adamw.py:198 */
     float neg_step_size;  /* float32(-(lr/bc))                      adamw.py:200 */

@@ -46,8 +46,9 @@ def make_scalars(lr: float, betas: Tuple[float, float], eps: float, weight_decay
     bias_correction_sqrt = (1 - beta2 ** step) ** (1 / 2)
     step_size = lr / bias_correction
     f32 = np.float32
-    # `tensor / python_float` on the GPU multiplies by the float32 reciprocal of the scalar
-    inv_bcs = f32(1.0) / f32(bias_correction_sqrt)
+    # `tensor / python_float` on the GPU multiplies by the reciprocal of the scalar, taken in
+    # double precision and then rounded to float32
+    inv_bcs = f32(1.0 / bias_correction_sqrt)
     apply_decay = weight_decay != 0
     return N.RtScalars(
         beta1=f32(beta1), one_m_beta1=f32(1 - beta1), beta2=f32(beta2), one_m_beta2=f32(1 - beta2),

@@ -135,8 +135,12 @@ class AdamW(Optimizer):
         return ids
 
     # -- step ----------------------------------------------------------------------
-    def step(self, closure=None, *, noise=None, debug_out=None):
+    def step(self, closure=None, *, noise=None, debug_out=None, grads=None):
         """One optimizer step (adamw.py:106-234).
+
+        ``grads``: optional ``{param: gradient}`` used instead of ``param.grad`` --
+        for gradients torch will not store in ``.grad`` (an fp32 gradient of a
+        bf16 param, a GPU gradient of a host-resident param).
 
         ``noise``: optional ``{param: (noise_p, noise_m, noise_v)}`` of int16 GPU
         tensors -- the explicit-noise test mode (every stepped bf16 array needs one).
@@ -163,9 +167,9 @@ class AdamW(Optimizer):
             for gi, group in enumerate(self.param_groups):
                 beta1, beta2 = group["betas"]
                 for p in group["params"]:
-                    if p.grad is None:
+                    grad = grads.get(p, p.grad) if grads is not None else p.grad
+                    if grad is None:
                         continue  # adamw.py:114: skipped, and its step count does not advance
-                    grad = p.grad
                     if grad.is_sparse:
                         raise RuntimeError("AdamW does not support sparse gradients")  # adamw.py:118-119
                     state = self.state[p]

@@ -1,0 +1,281 @@
+"""The ``AdamW`` class and the side entry points on the GPU: several steps
+against the reference's own op sequence, unbiasedness of the Philox rounding,
+grad-norm clip, centralization, copy_stochastic_.  Run with ``-m gpu``.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import torch_ops
+import ramtorch_amd
+from ramtorch_amd import _native as N
+from ramtorch_amd import functional as F
+
+pytestmark = pytest.mark.gpu
+HP0 = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
+
+
+def dev16(a, dt=torch.bfloat16):
+    return torch.from_numpy(a.view(np.int16).copy()).view(dt).cuda()
+
+
+def bits16(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def _make_params(shapes, seed, device="cuda"):
+    ps, grads = [], []
+    for i, shp in enumerate(shapes):
+        n = int(np.prod(shp)) if len(shp) else 1
+        p, g, _, _ = oracle.synth_inputs(n, seed + i)
+        ps.append(torch.nn.Parameter(dev16(p).view(shp).to(device)))
+        grads.append(dev16(g).view(shp))
+    return ps, grads
+
+
+def test_three_steps_match_the_reference_op_sequence():
+    """GPU params, GPU states, explicit noise: bit-exact against the ATen op
+    sequence of the reference (adamw.py:160-222) run on the same GPU."""
+    shapes = [(64, 48), (1000,), (3, 5, 7), ()]
+    ps, grads = _make_params(shapes, 100)
+    ref_p = [p.detach().clone() for p in ps]
+    opt = ramtorch_amd.AdamW([{"params": ps[:2]}, {"params": ps[2:], "lr": 5e-4, "weight_decay": 0.0}], lr=1e-3,
+                             storage_device="cuda")
+    ref_m = [torch.zeros_like(p) for p in ref_p]
+    ref_v = [torch.zeros_like(p) for p in ref_p]
+    for step in (1, 2, 3):
+        noise = {}
+        for i, p in enumerate(ps):
+            p.grad = (grads[i].float() * (1.0 + 0.1 * step)).bfloat16()
+            noise[p] = tuple(torch.randint(-32768, 32768, p.shape, dtype=torch.int16, device="cuda",
+                                           generator=torch.Generator("cuda").manual_seed(step * 10 + i * 3 + k))
+                             for k in range(3))
+        opt.step(noise=noise)
+        torch.cuda.synchronize()
+        for i, p in enumerate(ps):
+            grp = opt.param_groups[0 if i < 2 else 1]
+            torch_ops.reference_step_ops(ref_p[i], p.grad, ref_m[i], ref_v[i], lr=grp["lr"], betas=grp["betas"],
+                                         eps=grp["eps"], weight_decay=grp["weight_decay"], step=step, noise=noise[p])
+            assert torch.equal(p.detach(), ref_p[i]), f"step {step} param {i}"
+            assert torch.equal(opt.state[p]["ema"], ref_m[i]), f"step {step} ema {i}"
+            assert torch.equal(opt.state[p]["ema_squared"], ref_v[i]), f"step {step} ema_squared {i}"
+            assert opt.state[p]["step"] == step
+
+
+def test_skipped_and_sparse_gradients():
+    ps, grads = _make_params([(32, 8), (40,)], 200)
+    opt = ramtorch_amd.AdamW(ps, storage_device="cuda")
+    ps[0].grad = grads[0]
+    before = ps[1].detach().clone()
+    opt.step()
+    torch.cuda.synchronize()
+    assert opt.state[ps[0]]["step"] == 1 and opt.state[ps[1]]["step"] == 0  # adamw.py:114: no grad, no step
+    assert torch.equal(ps[1].detach(), before)
+    emb = torch.nn.Parameter(torch.zeros(10, 4, device="cuda"))
+    emb.grad = torch.sparse_coo_tensor(torch.tensor([[1], [2]]), torch.tensor([1.0]), (10, 4)).cuda()
+    with pytest.raises(RuntimeError, match="sparse"):
+        ramtorch_amd.AdamW([emb], storage_device="cuda").step()
+
+
+def test_lr_schedule_is_reread_every_step():
+    ps, grads = _make_params([(128,)], 300)
+    opt = ramtorch_amd.AdamW(ps, lr=1e-3, storage_device="cuda", seed=4)
+    sched = torch.optim.lr_scheduler.LambdaLR(opt, lambda e: 0.5 ** e)
+    p_ref, m_ref, v_ref = (bits16(ps[0]), np.zeros(128, np.uint16), np.zeros(128, np.uint16))
+    g = bits16(grads[0])
+    for step in (1, 2, 3):
+        ps[0].grad = grads[0]
+        opt.step()
+        lr = opt.param_groups[0]["lr"]
+        sc = oracle.scalars_from_hparams(lr, (0.9, 0.999), 1e-8, 1e-2, step)
+        oracle.step_tensor(p_ref, g, m_ref, v_ref, sc, seed=4, step=step, tensor_id=0)
+        sched.step()
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(bits16(ps[0]), p_ref, err_msg=f"step {step} lr {lr}")
+    assert opt.param_groups[0]["lr"] == pytest.approx(1e-3 * 0.125)
+
+
+def test_state_dict_resume_continues_bit_exactly():
+    ps, grads = _make_params([(300,), (16, 16)], 400)
+    a = ramtorch_amd.AdamW(ps, storage_device="cuda", seed=11)
+    for _ in range(2):
+        for p, g in zip(ps, grads):
+            p.grad = g
+        a.step()
+    sd = a.state_dict()
+    ps2 = [torch.nn.Parameter(p.detach().clone()) for p in ps]
+    b = ramtorch_amd.AdamW(ps2, storage_device="cuda", seed=11)
+    b.load_state_dict(sd)
+    for opt, params in ((a, ps), (b, ps2)):
+        for p, g in zip(params, grads):
+            p.grad = g
+        opt.step()
+    torch.cuda.synchronize()
+    for p, q in zip(ps, ps2):
+        assert torch.equal(p.detach(), q.detach())
+        assert torch.equal(a.state[p]["ema_squared"], b.state[q]["ema_squared"]) and b.state[q]["step"] == 3
+
+
+def test_non_contiguous_param_round_trips():
+    base = torch.nn.Parameter(dev16(oracle.synth_inputs(64 * 32, 500)[0]).view(64, 32).t())  # transposed view
+    assert not base.is_contiguous()
+    g = dev16(oracle.synth_inputs(64 * 32, 500)[1]).view(64, 32).t()
+    ref = torch.nn.Parameter(base.detach().contiguous())
+    o1 = ramtorch_amd.AdamW([base], storage_device="cuda", seed=2)
+    o2 = ramtorch_amd.AdamW([ref], storage_device="cuda", seed=2)
+    base.grad, ref.grad = g, g.contiguous()
+    o1.step(), o2.step()
+    torch.cuda.synchronize()
+    assert torch.equal(base.detach().contiguous(), ref.detach())
+
+
+def test_philox_rounding_is_unbiased_over_1e8_elements():
+    """Mean signed rounding error of each of p, m, v below 1e-3 bf16 ulp over 1e8 elements."""
+    n = 100_000_000
+    h = N.Handle(0)
+    gen = torch.Generator("cuda").manual_seed(1234)
+    P = (torch.randn(n, device="cuda", generator=gen) * 0.02).bfloat16()
+    G = (torch.randn(n, device="cuda", generator=gen) * 1e-3).bfloat16()
+    M = (torch.randn(n, device="cuda", generator=gen) * 1e-4).bfloat16()
+    V = ((torch.randn(n, device="cuda", generator=gen) * 1e-3) ** 2).bfloat16()
+    dbg = tuple(torch.empty(n, device="cuda") for _ in range(3))
+    e = F.Entry(p=P, g=G, m=M, v=V, step=100, scalars_idx=0, tensor_id=0, dbg=dbg)
+    F.step_resident(h, [e], [F.make_scalars(step=100, **HP0)], seed=1234, explicit_noise=False)
+    torch.cuda.synchronize()
+    for name, out, pre in zip("pmv", (P, M, V), dbg):
+        # one bf16 ulp at the magnitude of the fp32 value: 2^(exponent - 7)
+        ulp = torch.ldexp(torch.ones_like(pre), torch.frexp(pre)[1] - 8)
+        err = ((out.double() - pre.double()) / ulp.double())
+        err = err[pre != 0]
+        assert float(err.abs().max()) < 1.0 + 1e-9, name          # never further than one ulp
+        mean = float(err.mean())
+        assert abs(mean) < 1e-3, f"{name}: mean rounding error {mean:.3e} ulp"
+        assert 0.05 < float(err.std()) < 0.5, name                 # it does randomise
+    # the three arrays do not share noise: errors of p and m are uncorrelated
+    ep = (P.float() - dbg[0])[:10_000_000]
+    em = (M.float() - dbg[1])[:10_000_000]
+    c = torch.corrcoef(torch.stack([ep / ep.std(), em / em.std()]))[0, 1]
+    assert abs(float(c)) < 5e-3
+    h.close()
+
+
+def test_philox_noise_matches_oracle_stream_and_differs_between_steps_and_tensors():
+    n = 10_000
+    p, g, m, v = oracle.synth_inputs(n, 600)
+    h = N.Handle(0)
+    outs = {}
+    for step, tid, seed in ((5, 0, 1), (6, 0, 1), (5, 1, 1), (5, 0, 2)):
+        e = F.Entry(p=dev16(p), g=dev16(g), m=dev16(m), v=dev16(v), step=step, scalars_idx=0, tensor_id=tid)
+        F.step_resident(h, [e], [F.make_scalars(step=5, **HP0)], seed=seed, explicit_noise=False)
+        torch.cuda.synchronize()
+        outs[(step, tid, seed)] = bits16(e.p)
+        po, mo, vo = p.copy(), m.copy(), v.copy()
+        oracle.step_tensor(po, g, mo, vo, oracle.scalars_from_hparams(step=5, **HP0), seed=seed, step=step,
+                           tensor_id=tid)
+        np.testing.assert_array_equal(outs[(step, tid, seed)], po)
+    keys = list(outs)
+    for i in range(len(keys)):
+        for j in range(i + 1, len(keys)):
+            assert (outs[keys[i]] != outs[keys[j]]).mean() > 0.05
+    h.close()
+
+
+def test_grad_norm_clip_and_skip():
+    h = N.Handle(0)
+    rng = np.random.default_rng(0)
+    grads_np = [(rng.normal(0, 1e-3, n).astype(np.float32) * 1024) for n in (1, 1000, 8192 * 3 + 7, 250_000)]
+    grads = [torch.from_numpy(g).cuda() for g in grads_np] + [torch.zeros(0, device="cuda")]
+    grads.append(dev16(oracle.f32_to_bf16_rne(grads_np[1])))
+    out = F.grad_norm(h, grads, inv_loss_scale=1 / 1024, max_norm=0.01)
+    torch.cuda.synchronize()
+    want = sum(oracle.grad_sumsq(g, oracle.DT_F32, 1 / 1024) for g in grads_np)
+    want += oracle.grad_sumsq(oracle.f32_to_bf16_rne(grads_np[1]), oracle.DT_BF16, 1 / 1024)
+    total = float(out[0])
+    assert total == pytest.approx(want ** 0.5, rel=1e-6)
+    assert np.float32(out[1].item()) == oracle.clip_coef(np.float32(total), 0.01)
+    assert out.view(torch.int32)[2].item() == 0
+    again = F.grad_norm(h, grads, inv_loss_scale=1 / 1024, max_norm=0.01)
+    assert torch.equal(out[:2], again[:2])  # deterministic reduction order
+    grads[2][5] = float("inf")
+    bad = F.grad_norm(h, grads, inv_loss_scale=1 / 1024, max_norm=0.01)
+    assert bad.view(torch.int32)[2].item() == 1 and float(bad[1]) == 1.0
+    h.close()
+
+
+def test_optimizer_with_loss_scale_and_max_grad_norm():
+    """Config-4 layout: bf16 p, fp32 grads pre-scaled by 1024, global clip to 1.0."""
+    shapes = [(256, 64), (512,)]
+    ps, _ = _make_params(shapes, 700)
+    opt = ramtorch_amd.AdamW(ps, storage_device="cuda", seed=8, loss_scale=1024.0, max_grad_norm=1.0, **HP0)
+    gnp = [np.random.default_rng(i).normal(0, 0.05, int(np.prod(s))).astype(np.float32) * 1024 for i, s in
+           enumerate(shapes)]
+    gmap = {p: torch.from_numpy(g).cuda().view(p.shape) for p, g in zip(ps, gnp)}  # fp32 grads of bf16 params
+    before = [bits16(p) for p in ps]
+    opt.step(grads=gmap)
+    torch.cuda.synchronize()
+    total = float(opt.last_grad_norm[0])
+    coef = np.float32(opt.last_grad_norm[1].item())
+    assert total == pytest.approx(sum(oracle.grad_sumsq(g, oracle.DT_F32, 1 / 1024) for g in gnp) ** 0.5, rel=1e-6)
+    assert coef < 1.0
+    sc = oracle.scalars_from_hparams(step=1, inv_loss_scale=1 / 1024, apply_clip=True, **HP0)
+    for i, (p, g) in enumerate(zip(ps, gnp)):
+        n = g.size
+        po, mo, vo = before[i].copy(), np.zeros(n, np.uint16), np.zeros(n, np.uint16)
+        oracle.step_tensor(po, g, mo, vo, sc, g_dtype=oracle.DT_F32, clip_coef=coef, seed=8, step=1, tensor_id=i)
+        np.testing.assert_array_equal(bits16(p), po)
+        np.testing.assert_array_equal(bits16(opt.state[p]["ema_squared"]), vo)
+    # a non-finite gradient skips the whole update
+    snap = [p.detach().clone() for p in ps]
+    gmap[ps[0]][0, 0] = float("nan")
+    opt.step(grads=gmap)
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b.detach()) for a, b in zip(snap, ps))
+    assert opt.last_grad_norm.view(torch.int32)[2].item() == 1
+
+
+@pytest.mark.parametrize("shape", [(37, 24), (4, 3, 10), (129,), ()])
+def test_centralization(shape):
+    n = int(np.prod(shape)) if len(shape) else 1
+    p, g, _, _ = oracle.synth_inputs(n, 800)
+    P = torch.nn.Parameter(dev16(p).view(shape))
+    P.grad = dev16(g).view(shape)
+    opt = ramtorch_amd.AdamW([P], storage_device="cuda", seed=3, centralization=0.5, **HP0)
+    opt.step()
+    torch.cuda.synchronize()
+    rows = shape[0] if len(shape) >= 2 else 1
+    row_len = n // rows
+    h = N.Handle(0)
+    means = F.row_means(h, P.grad.contiguous(), rows, row_len).cpu().numpy()
+    np.testing.assert_allclose(means, oracle.row_means(g, rows, row_len), rtol=2e-6, atol=1e-9)
+    # same means in, bit-exact out: g' = g - fl(mean * c), then the usual update
+    g32 = oracle.bf16_to_f32(g) - (np.repeat(means, row_len) * np.float32(0.5)).astype(np.float32)
+    po, mo, vo = p.copy(), np.zeros(n, np.uint16), np.zeros(n, np.uint16)
+    oracle.step_tensor(po, g32.astype(np.float32), mo, vo, oracle.scalars_from_hparams(step=1, **HP0),
+                       g_dtype=oracle.DT_F32, seed=3, step=1, tensor_id=0)
+    np.testing.assert_array_equal(bits16(P), po)
+    # and against torch's own formulation (adamw.py:179-184), within the mean's tolerance
+    gt = P.grad.float()
+    gt = gt - gt.mean(dim=tuple(range(1, gt.dim())), keepdim=True) * 0.5
+    np.testing.assert_allclose(g32.reshape(shape), gt.cpu().numpy(), rtol=1e-5, atol=1e-9)
+    h.close()
+
+
+def test_copy_stochastic():
+    n = 100_003
+    src = torch.randn(n, device="cuda") * 0.02
+    noise = torch.randint(-32768, 32768, (n,), dtype=torch.int16, device="cuda")
+    tgt = torch.empty(n, dtype=torch.bfloat16, device="cuda")
+    ramtorch_amd.copy_stochastic_(tgt, src, noise=noise)
+    torch.cuda.synchronize()
+    want = oracle.sr_copy(src.cpu().numpy(), noise=noise.cpu().numpy())
+    np.testing.assert_array_equal(bits16(tgt), want)
+    ref = torch.empty_like(tgt)
+    torch_ops.sr_write_(ref, src, torch_ops.noise_to_i32(noise))   # the reference's integer ops on the GPU
+    assert torch.equal(ref, tgt)
+    ramtorch_amd.copy_stochastic_(tgt, src, seed=42)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(bits16(tgt), oracle.sr_copy(src.cpu().numpy(), seed=42))
+    cpu_tgt = torch.empty(n, dtype=torch.bfloat16)
+    ramtorch_amd.copy_stochastic_(cpu_tgt, src, seed=42)
+    assert torch.equal(cpu_tgt, tgt.cpu())

@@ -1,0 +1,324 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle and with
+torch's own GPU kernels.  Needs an MI355X: run with ``-m gpu``.
+
+Bar: bit-exact for every bf16 result and for the fp32 values before rounding.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import torch_ops
+from ramtorch_amd import _native as N
+from ramtorch_amd import functional as F
+
+pytestmark = pytest.mark.gpu
+
+HP0 = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
+_NP2T = {np.dtype(np.uint16): torch.int16, np.dtype(np.float32): torch.float32}
+
+
+@pytest.fixture(scope="module")
+def handle():
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    h = N.Handle(0)
+    yield h
+    torch.cuda.synchronize()
+    h.close()
+
+
+def dev16(a, dt=torch.bfloat16):
+    """uint16 bit patterns -> GPU tensor of a 16-bit dtype."""
+    return torch.from_numpy(a.view(np.int16).copy()).view(dt).cuda()
+
+
+def bits16(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def bits32(t):
+    return t.detach().cpu().contiguous().numpy().view(np.uint32)
+
+
+def run_both(handle, p, g, m, v, *, hp=HP0, step=10, noise=None, seed=1234, tensor_id=0, debug=True,
+             g_dtype=oracle.DT_BF16, p_dtype=oracle.DT_BF16, m_dtype=oracle.DT_BF16, v_dtype=oracle.DT_BF16,
+             inv_loss_scale=1.0, clip_coef=None):
+    """One tensor through the HIP library and through the oracle; returns both result sets."""
+    tdt = {oracle.DT_BF16: torch.bfloat16, oracle.DT_F16: torch.float16}
+
+    def up(a, code):
+        return torch.from_numpy(a.copy()).cuda() if code == oracle.DT_F32 else dev16(a, tdt[code])
+
+    P, G, M, V = up(p, p_dtype), up(g, g_dtype), up(m, m_dtype), up(v, v_dtype)
+    n = p.size
+    NZ = None if noise is None else tuple(torch.from_numpy(z.view(np.int16).copy()).cuda() for z in noise)
+    dbg = tuple(torch.full((n,), float("nan"), device="cuda") for _ in range(3)) if debug else None
+    e = F.Entry(p=P, g=G, m=M, v=V, step=step, scalars_idx=0, tensor_id=tensor_id, noise=NZ, dbg=dbg)
+    sc = F.make_scalars(step=step, inv_loss_scale=inv_loss_scale, **hp)
+    coef_t = None if clip_coef is None else torch.tensor([clip_coef], dtype=torch.float32, device="cuda")
+    F.step_resident(handle, [e], [sc], seed=seed, explicit_noise=noise is not None, clip_coef=coef_t)
+    torch.cuda.synchronize()
+
+    po, mo, vo = p.copy(), m.copy(), v.copy()
+    sco = oracle.scalars_from_hparams(step=step, inv_loss_scale=inv_loss_scale, apply_clip=clip_coef is not None, **hp)
+    d = oracle.step_tensor(po, g, mo, vo, sco, p_dtype=p_dtype, g_dtype=g_dtype, m_dtype=m_dtype, v_dtype=v_dtype,
+                           clip_coef=1.0 if clip_coef is None else clip_coef, noise=noise, seed=seed, step=step,
+                           tensor_id=tensor_id, debug=True)
+    got = [bits32(t) if t.dtype == torch.float32 else bits16(t) for t in (P, M, V)]
+    want = [a.view(np.uint32) if a.dtype == np.float32 else a for a in (po, mo, vo)]
+    return got, want, (None if dbg is None else [bits32(t) for t in dbg]), [x.view(np.uint32) for x in d]
+
+
+def assert_same(got, want, dbg, pre, what=""):
+    for name, a, b in zip("pmv", got, want):
+        np.testing.assert_array_equal(a, b, err_msg=f"{what} {name} (stored)")
+    if dbg is not None:
+        for name, a, b in zip("pmv", dbg, pre):
+            np.testing.assert_array_equal(a, b, err_msg=f"{what} {name} (fp32 before rounding)")
+
+
+# ---- the flavour pin: torch's GPU kernels are the reference's arithmetic -----------------
+def test_reference_flavour_is_what_torch_gpu_kernels_compute():
+    n = 1 << 20
+    p, g, m, v = oracle.synth_inputs(n, 1234)
+    noise = oracle.synth_noise(n, 1234)
+    P, G, M, V = dev16(p), dev16(g), dev16(m), dev16(v)
+    NZ = [torch.from_numpy(z.view(np.int16).copy()).cuda() for z in noise]
+    p32, m32, v32 = torch_ops.reference_step_ops(P, G, M, V, step=10, noise=NZ, **HP0)
+    torch.cuda.synchronize()
+    sc = oracle.scalars_from_hparams(step=10, **HP0)
+    po, mo, vo = p.copy(), m.copy(), v.copy()
+    d = oracle.step_tensor(po, g, mo, vo, sc, noise=noise, flavour=oracle.REFERENCE_FLAVOUR, debug=True)
+    for name, t, a in zip("pmv", (p32, m32, v32), d):
+        np.testing.assert_array_equal(bits32(t), a.view(np.uint32), err_msg=f"fp32 {name}")
+    for name, t, a in zip("pmv", (P, M, V), (po, mo, vo)):
+        np.testing.assert_array_equal(bits16(t), a, err_msg=f"bf16 {name}")
+    # and the CPU flavour is measurably different, so the pin is sharp
+    d2 = oracle.step_tensor(p.copy(), g, m.copy(), v.copy(), sc, noise=noise, flavour=oracle.TORCH_CPU_FLAVOUR,
+                            debug=True)
+    assert (d2[0].view(np.uint32) != bits32(p32)).sum() > 0
+
+
+# ---- config 0: one 4096 x 4096 weight, explicit noise, bit-exact ----------------------------
+def test_config0_bit_exact_against_oracle_and_torch_gpu_ops(handle):
+    n = 4096 * 4096
+    p, g, m, v = oracle.synth_inputs(n, 1234)
+    noise = oracle.synth_noise(n, 1234)
+    got, want, dbg, pre = run_both(handle, p, g, m, v, noise=noise, step=10)
+    assert_same(got, want, dbg, pre, "config0")
+    # fast path (no debug outputs) gives the same stored bits
+    got2, _, _, _ = run_both(handle, p, g, m, v, noise=noise, step=10, debug=False)
+    assert_same(got2, want, None, None, "config0 fast path")
+    # the reference's own op sequence on the GPU
+    P, G, M, V = (dev16(a).view(4096, 4096) for a in (p, g, m, v))
+    NZ = [torch.from_numpy(z.view(np.int16).copy()).cuda().view(4096, 4096) for z in noise]
+    p32, m32, v32 = torch_ops.reference_step_ops(P, G, M, V, step=10, noise=NZ, **HP0)
+    for name, t, a in zip("pmv", (P, M, V), got2):
+        np.testing.assert_array_equal(bits16(t).ravel(), a, err_msg=f"torch GPU ops vs HIP {name}")
+    for name, t, a in zip("pmv", (p32, m32, v32), dbg):
+        np.testing.assert_array_equal(bits32(t).ravel(), a, err_msg=f"torch GPU ops vs HIP fp32 {name}")
+
+
+# ---- sizes: empty, tiny, ragged, chunk boundaries -------------------------------------------
+@pytest.mark.parametrize("n", [1, 7, 8, 9, 2047, 2048, 8191, 8192, 8193, 3 * 8192 + 5, 100_003])
+@pytest.mark.parametrize("mode", ["explicit", "philox"])
+def test_sizes_and_tails(handle, n, mode):
+    p, g, m, v = oracle.synth_inputs(n, n)
+    noise = oracle.synth_noise(n, n) if mode == "explicit" else None
+    for debug in (True, False):
+        got, want, dbg, pre = run_both(handle, p, g, m, v, noise=noise, step=3, tensor_id=5, debug=debug)
+        assert_same(got, want, dbg, pre, f"n={n} {mode}")
+
+
+def test_empty_inputs(handle):
+    F.step_resident(handle, [], [], seed=0, explicit_noise=False)
+    z = torch.zeros(0, dtype=torch.bfloat16, device="cuda")
+    e = F.Entry(p=z, g=z.clone(), m=z.clone(), v=z.clone(), step=1, scalars_idx=0, tensor_id=0)
+    F.step_resident(handle, [e], [F.make_scalars(step=1, **HP0)], seed=0, explicit_noise=False)
+    torch.cuda.synchronize()
+
+
+def test_unaligned_views(handle):
+    # a view that starts 2 bytes into an allocation: no 128-bit access is legal
+    n = 5000
+    p, g, m, v = oracle.synth_inputs(n, 21)
+    base = [torch.zeros(n + 8, dtype=torch.bfloat16, device="cuda") for _ in range(4)]
+    views = []
+    for b, a, off in zip(base, (p, g, m, v), (1, 3, 0, 5)):
+        b[off:off + n] = dev16(a)
+        views.append(b[off:off + n])
+    e = F.Entry(p=views[0], g=views[1], m=views[2], v=views[3], step=10, scalars_idx=0, tensor_id=1)
+    F.step_resident(handle, [e], [F.make_scalars(step=10, **HP0)], seed=7, explicit_noise=False)
+    torch.cuda.synchronize()
+    po, mo, vo = p.copy(), m.copy(), v.copy()
+    oracle.step_tensor(po, g, mo, vo, oracle.scalars_from_hparams(step=10, **HP0), seed=7, step=10, tensor_id=1)
+    for name, t, a in zip("pmv", (views[0], views[2], views[3]), (po, mo, vo)):
+        np.testing.assert_array_equal(bits16(t), a, err_msg=name)
+    # nothing outside the views was written
+    assert float(base[0][0]) == 0 and not base[0][n + 1:].any() and not base[3][:5].any()
+
+
+# ---- value edge cases -------------------------------------------------------------------------
+def test_edge_values(handle):
+    import itertools
+    vals = [0x0000, 0x8000, 0x0001, 0x8001, 0x007F, 0x0080, 0x0100, 0x3F80, 0xBF80, 0x7F7F, 0xFF7F, 0x4000, 0x3F00,
+            0x1234, 0x9234, 0x2B00, 0x6000, 0x0F00, 0x3DCC, 0x3A83, 0x7F80, 0xFF80]
+    combos = list(itertools.product(range(len(vals)), repeat=2))
+    p = np.array([vals[a] for a, b in combos], np.uint16)
+    g = np.array([vals[b] for a, b in combos], np.uint16)
+    m = np.array([vals[(a + b) % len(vals)] for a, b in combos], np.uint16)
+    v = np.array([vals[(a * 7 + b) % len(vals)] & 0x7FFF for a, b in combos], np.uint16)
+    noise = oracle.synth_noise(p.size, 99)
+    got, want, dbg, pre = run_both(handle, p, g, m, v, noise=noise)
+    # NaN payloads are not part of the contract; everything else is bit-exact
+    for name, a, b, d_, q in zip("pmv", got, want, dbg, pre):
+        ok = ~np.isnan(q.view(np.float32))
+        np.testing.assert_array_equal(d_[ok], q[ok], err_msg=f"fp32 {name}")
+        np.testing.assert_array_equal(a[ok], b[ok], err_msg=f"bf16 {name}")
+        assert np.isnan(d_.view(np.float32)[~ok]).all()
+
+
+# ---- hyper-parameters and steps -------------------------------------------------------------------
+@pytest.mark.parametrize("hp,step", [
+    (dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01), 1),
+    (dict(lr=3e-4, betas=(0.95, 0.99), eps=1e-6, weight_decay=0.0), 100),
+    (dict(lr=2.5e-3, betas=(0.8, 0.9999), eps=1e-10, weight_decay=0.1), 5000),
+    (dict(lr=1e-4, betas=(0.0, 0.5), eps=1e-8, weight_decay=1.0), 2),
+])
+def test_hyperparameters(handle, hp, step):
+    n = 50_000
+    p, g, m, v = oracle.synth_inputs(n, step)
+    got, want, dbg, pre = run_both(handle, p, g, m, v, hp=hp, step=step, noise=oracle.synth_noise(n, step))
+    assert_same(got, want, dbg, pre, f"{hp} step {step}")
+
+
+# ---- dtype combinations (fp32 params / states are stored without rounding) ------------------------
+@pytest.mark.parametrize("p_dt,g_dt,m_dt,v_dt", [
+    (oracle.DT_BF16, oracle.DT_F32, oracle.DT_BF16, oracle.DT_F32),   # config 4 layout
+    (oracle.DT_F32, oracle.DT_F32, oracle.DT_F32, oracle.DT_F32),
+    (oracle.DT_BF16, oracle.DT_F16, oracle.DT_BF16, oracle.DT_BF16),
+    (oracle.DT_F32, oracle.DT_BF16, oracle.DT_BF16, oracle.DT_BF16),
+    (oracle.DT_BF16, oracle.DT_BF16, oracle.DT_F32, oracle.DT_BF16),
+])
+@pytest.mark.parametrize("mode", ["explicit", "philox"])
+def test_dtype_combinations(handle, p_dt, g_dt, m_dt, v_dt, mode):
+    n = 20_000 + 3
+    p, g, m, v = oracle.synth_inputs(n, 31)
+
+    def conv(a, dt):
+        if dt == oracle.DT_F32:
+            return (oracle.bf16_to_f32(a) * np.float32(1.0009765625)).astype(np.float32)  # not bf16-exact
+        if dt == oracle.DT_F16:
+            return oracle.bf16_to_f32(a).astype(np.float16).view(np.uint16)
+        return a
+    p, g, m, v = conv(p, p_dt), conv(g, g_dt), conv(m, m_dt), conv(v, v_dt)
+    noise = oracle.synth_noise(n, 31) if mode == "explicit" else None
+    for debug in (True, False):
+        got, want, dbg, pre = run_both(handle, p, g, m, v, noise=noise, p_dtype=p_dt, g_dtype=g_dt, m_dtype=m_dt,
+                                       v_dtype=v_dt, debug=debug)
+        assert_same(got, want, dbg, pre, f"dtypes {p_dt}{g_dt}{m_dt}{v_dt} {mode}")
+
+
+def test_loss_scale_and_clip_coefficient(handle):
+    n = 30_000
+    p, g, m, v = oracle.synth_inputs(n, 41)
+    g32 = (oracle.bf16_to_f32(g) * np.float32(1024)).astype(np.float32)
+    v32 = oracle.bf16_to_f32(v).copy()
+    got, want, dbg, pre = run_both(handle, p, g32, m, v32, g_dtype=oracle.DT_F32, v_dtype=oracle.DT_F32,
+                                   inv_loss_scale=1.0 / 1024, clip_coef=0.37, step=100)
+    assert_same(got, want, dbg, pre, "loss scale + clip")
+
+
+# ---- many tensors in one launch ---------------------------------------------------------------------
+def test_multi_tensor_launch_with_groups_and_steps(handle):
+    rng = np.random.default_rng(5)
+    lens = [int(x) for x in np.exp(rng.uniform(0, np.log(4096), 300)).astype(np.int64).clip(1, 4096)]
+    lens += [0, 8192, 8192 * 2 + 1, 1, 65_537]
+    hps = [HP0, dict(lr=3e-4, betas=(0.95, 0.99), eps=1e-6, weight_decay=0.0)]
+    scal, sco, entries, inputs = [], [], [], []
+    for gi, hp in enumerate(hps):
+        for st in (4, 9):
+            scal.append(F.make_scalars(step=st, **hp))
+            sco.append((oracle.scalars_from_hparams(step=st, **hp), st))
+    for i, n in enumerate(lens):
+        p, g, m, v = oracle.synth_inputs(n, 1000 + i)
+        si = i % len(scal)
+        P, G, M, V = dev16(p), dev16(g), dev16(m), dev16(v)
+        entries.append(F.Entry(p=P, g=G, m=M, v=V, step=sco[si][1], scalars_idx=si, tensor_id=i))
+        inputs.append((p, g, m, v, si))
+    F.step_resident(handle, entries, scal, seed=99, explicit_noise=False)
+    torch.cuda.synchronize()
+    for i, (e, (p, g, m, v, si)) in enumerate(zip(entries, inputs)):
+        po, mo, vo = p.copy(), m.copy(), v.copy()
+        oracle.step_tensor(po, g, mo, vo, sco[si][0], seed=99, step=sco[si][1], tensor_id=i)
+        for name, t, a in zip("pmv", (e.p, e.m, e.v), (po, mo, vo)):
+            np.testing.assert_array_equal(bits16(t), a, err_msg=f"tensor {i} (n={lens[i]}) {name}")
+
+
+def test_mixed_dtype_tensors_in_one_call(handle):
+    n = 10_000
+    p, g, m, v = oracle.synth_inputs(n, 61)
+    sc, sco = F.make_scalars(step=2, **HP0), oracle.scalars_from_hparams(step=2, **HP0)
+    e0 = F.Entry(p=dev16(p), g=dev16(g), m=dev16(m), v=dev16(v), step=2, scalars_idx=0, tensor_id=0)
+    p32 = oracle.bf16_to_f32(p).copy()
+    e1 = F.Entry(p=torch.from_numpy(p32.copy()).cuda(), g=dev16(g), m=dev16(m), v=dev16(v), step=2, scalars_idx=0,
+                 tensor_id=1)
+    F.step_resident(handle, [e0, e1], [sc], seed=3, explicit_noise=False)
+    torch.cuda.synchronize()
+    a = [p.copy(), m.copy(), v.copy()]
+    oracle.step_tensor(a[0], g, a[1], a[2], sco, seed=3, step=2, tensor_id=0)
+    b = [p32.copy(), m.copy(), v.copy()]
+    oracle.step_tensor(b[0], g, b[1], b[2], sco, p_dtype=oracle.DT_F32, seed=3, step=2, tensor_id=1)
+    np.testing.assert_array_equal(bits16(e0.p), a[0])
+    np.testing.assert_array_equal(bits32(e1.p), b[0].view(np.uint32))
+    np.testing.assert_array_equal(bits16(e1.m), b[1])
+
+
+# ---- pieces of a tensor draw the same noise as the whole -----------------------------------------
+def test_elem_offset_pieces_equal_whole(handle):
+    n = 40_000
+    p, g, m, v = oracle.synth_inputs(n, 71)
+    sc = F.make_scalars(step=6, **HP0)
+    whole = F.Entry(p=dev16(p), g=dev16(g), m=dev16(m), v=dev16(v), step=6, scalars_idx=0, tensor_id=9)
+    F.step_resident(handle, [whole], [sc], seed=5, explicit_noise=False)
+    P, G, M, V = dev16(p), dev16(g), dev16(m), dev16(v)
+    cuts = [0, 8, 8200, 24_000, n]
+    pieces = [F.Entry(p=P[a:b], g=G[a:b], m=M[a:b], v=V[a:b], step=6, scalars_idx=0, tensor_id=9, elem_offset=a)
+              for a, b in zip(cuts[:-1], cuts[1:])]
+    F.step_resident(handle, pieces, [sc], seed=5, explicit_noise=False)
+    torch.cuda.synchronize()
+    assert torch.equal(whole.p, P) and torch.equal(whole.m, M) and torch.equal(whole.v, V)
+
+
+# ---- skip flag ----------------------------------------------------------------------------------------
+def test_skip_flag_leaves_everything_untouched(handle):
+    n = 9000
+    p, g, m, v = oracle.synth_inputs(n, 81)
+    e = F.Entry(p=dev16(p), g=dev16(g), m=dev16(m), v=dev16(v), step=1, scalars_idx=0, tensor_id=0)
+    skip = torch.ones(1, dtype=torch.int32, device="cuda")
+    F.step_resident(handle, [e], [F.make_scalars(step=1, **HP0)], seed=0, explicit_noise=False, skip=skip)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(bits16(e.p), p)
+    np.testing.assert_array_equal(bits16(e.m), m)
+    skip.zero_()
+    F.step_resident(handle, [e], [F.make_scalars(step=1, **HP0)], seed=0, explicit_noise=False, skip=skip)
+    torch.cuda.synchronize()
+    assert (bits16(e.m) != m).any()
+
+
+# ---- argument errors come back as error codes, not crashes ------------------------------------------------
+def test_bad_arguments_are_rejected(handle):
+    z = torch.zeros(16, dtype=torch.bfloat16, device="cuda")
+    e = F.Entry(p=z, g=z.clone(), m=z.clone(), v=z.clone(), step=1, scalars_idx=3, tensor_id=0)
+    with pytest.raises(N.NativeError, match="scalars_idx"):
+        F.step_resident(handle, [e], [F.make_scalars(step=1, **HP0)], seed=0, explicit_noise=False)
+    e.scalars_idx = 0
+    with pytest.raises(N.NativeError, match="explicit noise"):
+        F.step_resident(handle, [e], [F.make_scalars(step=1, **HP0)], seed=0, explicit_noise=True)
+    e.elem_offset = 4
+    with pytest.raises(N.NativeError, match="elem_offset"):
+        F.step_resident(handle, [e], [F.make_scalars(step=1, **HP0)], seed=0, explicit_noise=False)
+    e.elem_offset = 0
+    e.tensor_id = 1 << 30
+    with pytest.raises(N.NativeError, match="tensor_id"):
+        F.step_resident(handle, [e], [F.make_scalars(step=1, **HP0)], seed=0, explicit_noise=False)

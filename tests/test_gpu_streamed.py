@@ -1,0 +1,142 @@
+"""The host-resident (streamed) path: params / states in pinned host memory,
+chunked H2D -> update -> D2H.  Results must be bit-identical to the resident
+path and to the oracle, whatever the chunk size.  Run with ``-m gpu``.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import ramtorch_amd
+from ramtorch_amd import _native as N
+from ramtorch_amd import functional as F
+
+pytestmark = pytest.mark.gpu
+HP0 = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
+
+
+def host16(a, pin=True):
+    t = torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16)
+    return t.pin_memory() if pin else t
+
+
+def dev16(a):
+    return torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16).cuda()
+
+
+def bits16(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+@pytest.fixture(scope="module")
+def handle():
+    h = N.Handle(0)
+    yield h
+    torch.cuda.synchronize()
+    h.close()
+
+
+LENS = [1, 5, 8, 4096, 8191, 8193, 30_011, 16, 100_000, 0, 7]
+
+
+@pytest.mark.parametrize("chunk_elems", [8, 64, 4096, 8192, 65_536, 1 << 22])
+def test_streamed_equals_oracle_for_any_chunk_size(handle, chunk_elems):
+    sc, sco = F.make_scalars(step=10, **HP0), oracle.scalars_from_hparams(step=10, **HP0)
+    entries, inputs = [], []
+    lens = [n for n in LENS if n < 10_000] if chunk_elems < 64 else LENS  # keep the call count sane
+    for i, n in enumerate(lens):
+        p, g, m, v = oracle.synth_inputs(n, 50 + i)
+        entries.append(F.Entry(p=host16(p), g=dev16(g), m=host16(m), v=host16(v), step=10, scalars_idx=0,
+                               tensor_id=i))
+        inputs.append((p, g, m, v))
+    F.step_streamed(handle, entries, [sc], seed=77, explicit_noise=False, chunk_elems=chunk_elems)
+    # no synchronisation here on purpose: host memory must be final when the call returns
+    for i, (e, (p, g, m, v)) in enumerate(zip(entries, inputs)):
+        po, mo, vo = p.copy(), m.copy(), v.copy()
+        oracle.step_tensor(po, g, mo, vo, sco, seed=77, step=10, tensor_id=i)
+        for name, t, a in zip("pmv", (e.p, e.m, e.v), (po, mo, vo)):
+            np.testing.assert_array_equal(t.view(torch.int16).numpy().view(np.uint16), a,
+                                          err_msg=f"chunk {chunk_elems} tensor {i} (n={lens[i]}) {name}")
+    stats = handle.streamed_stats()
+    total = sum(lens)
+    assert stats["bytes_h2d"] == 6 * total and stats["bytes_d2h"] == 6 * total
+
+
+def test_streamed_mixed_residency_and_dtypes(handle):
+    """GPU params with host states (the constructor's default layout), host
+    unpinned gradients, fp32 state on the host, explicit noise."""
+    n = 50_000
+    p, g, m, v = oracle.synth_inputs(n, 90)
+    noise = oracle.synth_noise(n, 90)
+    NZ = tuple(torch.from_numpy(z.view(np.int16).copy()).cuda() for z in noise)
+    sc, sco = F.make_scalars(step=3, **HP0), oracle.scalars_from_hparams(step=3, **HP0)
+    v32 = oracle.bf16_to_f32(v).copy()
+    e0 = F.Entry(p=dev16(p), g=dev16(g), m=host16(m), v=host16(v), step=3, scalars_idx=0, tensor_id=0, noise=NZ)
+    e1 = F.Entry(p=host16(p), g=host16(g, pin=False), m=host16(m), v=torch.from_numpy(v32.copy()).pin_memory(),
+                 step=3, scalars_idx=0, tensor_id=1, noise=NZ)
+    F.step_streamed(handle, [e0, e1], [sc], seed=0, explicit_noise=True, chunk_elems=16_384)
+    torch.cuda.synchronize()
+    a = [p.copy(), m.copy(), v.copy()]
+    oracle.step_tensor(a[0], g, a[1], a[2], sco, noise=noise)
+    for name, t, w in zip("pmv", (e0.p, e0.m, e0.v), a):
+        np.testing.assert_array_equal(bits16(t), w, err_msg=f"e0 {name}")
+    b = [p.copy(), m.copy(), v32.copy()]
+    oracle.step_tensor(b[0], g, b[1], b[2], sco, v_dtype=oracle.DT_F32, noise=noise)
+    np.testing.assert_array_equal(bits16(e1.p), b[0])
+    np.testing.assert_array_equal(bits16(e1.m), b[1])
+    np.testing.assert_array_equal(e1.v.numpy().view(np.uint32), b[2].view(np.uint32))
+
+
+def test_streamed_and_resident_agree_bit_for_bit(handle):
+    n = 300_000
+    p, g, m, v = oracle.synth_inputs(n, 95)
+    sc = F.make_scalars(step=42, **HP0)
+    r = F.Entry(p=dev16(p), g=dev16(g), m=dev16(m), v=dev16(v), step=42, scalars_idx=0, tensor_id=4)
+    F.step_resident(handle, [r], [sc], seed=5, explicit_noise=False)
+    s = F.Entry(p=host16(p), g=dev16(g), m=host16(m), v=host16(v), step=42, scalars_idx=0, tensor_id=4)
+    F.step_streamed(handle, [s], [sc], seed=5, explicit_noise=False, chunk_elems=40_000)
+    torch.cuda.synchronize()
+    for a, b in ((r.p, s.p), (r.m, s.m), (r.v, s.v)):
+        assert torch.equal(a.cpu(), b)
+
+
+def test_optimizer_default_layout_cpu_params_and_pinned_states():
+    """The reference's offload flow: pinned CPU bf16 params (as ramtorch.Linear
+    creates them), CPU gradients, pinned CPU states, several steps."""
+    shapes = [(128, 96), (96,), (33, 7)]
+    ps, gs, refs = [], [], []
+    for i, shp in enumerate(shapes):
+        n = int(np.prod(shp))
+        p, g, _, _ = oracle.synth_inputs(n, 900 + i)
+        t = torch.nn.Parameter(host16(p).view(shp))
+        t.is_ramtorch = True
+        ps.append(t)
+        gs.append(g)
+        refs.append([p.copy(), np.zeros(n, np.uint16), np.zeros(n, np.uint16)])
+    opt = ramtorch_amd.AdamW(ps, seed=21, stream_chunk_bytes=16_384, **HP0)
+    assert all(opt.state[p]["ema"].is_pinned() and opt.state[p]["ema"].device.type == "cpu" for p in ps)
+    for step in (1, 2, 3):
+        for p, g in zip(ps, gs):
+            p.grad = host16(g, pin=False).view(p.shape)        # Linear.backward leaves CPU grads
+        opt.step()
+        sco = oracle.scalars_from_hparams(step=step, **HP0)
+        for i, (p, g) in enumerate(zip(ps, gs)):
+            oracle.step_tensor(refs[i][0], g, refs[i][1], refs[i][2], sco, seed=21, step=step, tensor_id=i)
+            np.testing.assert_array_equal(bits16(p), refs[i][0], err_msg=f"step {step} param {i}")
+            np.testing.assert_array_equal(bits16(opt.state[p]["ema"]), refs[i][1])
+            np.testing.assert_array_equal(bits16(opt.state[p]["ema_squared"]), refs[i][2])
+    assert all(p.is_pinned() for p in ps)  # params were updated in place
+
+
+def test_optimizer_gpu_params_with_default_cpu_states():
+    n = 20_000
+    p, g, _, _ = oracle.synth_inputs(n, 950)
+    P = torch.nn.Parameter(dev16(p))
+    P.grad = dev16(g)
+    opt = ramtorch_amd.AdamW([P], seed=1, **HP0)          # storage_device defaults to "cpu"
+    opt.step()
+    po, mo, vo = p.copy(), np.zeros(n, np.uint16), np.zeros(n, np.uint16)
+    oracle.step_tensor(po, g, mo, vo, oracle.scalars_from_hparams(step=1, **HP0), seed=1, step=1, tensor_id=0)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(bits16(P), po)
+    np.testing.assert_array_equal(bits16(opt.state[P]["ema"]), mo)

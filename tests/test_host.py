@@ -1,0 +1,208 @@
+"""Host-side logic and the C-ABI surface.  No GPU needed, no compute calls."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import ramtorch_amd
+from ramtorch_amd import _native as N
+from ramtorch_amd import functional as F
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "ramtorch_sr_adamw.h")
+
+
+# ---- the shared library and its header ---------------------------------------------------
+def test_library_loads_and_exports_every_declared_symbol():
+    L = N.lib()
+    assert L.rt_version() == N.ABI_VERSION
+    text = open(HEADER).read()
+    declared = set(re.findall(r"^\s*(?:int|const char\*)\s+(rt_\w+)\s*\(", text, flags=re.M))
+    assert declared == set(N.EXPORTS), declared ^ set(N.EXPORTS)
+    for name in declared:
+        assert hasattr(L, name), f"{name} declared in the header but not exported"
+
+
+def test_header_compiles_as_c_and_layouts_agree(tmp_path):
+    src = tmp_path / "layout.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <stddef.h>\n#include "ramtorch_sr_adamw.h"\n'
+        "int main(void){\n"
+        'printf("%zu %zu\\n", sizeof(rt_scalars), sizeof(rt_tensor_desc));\n'
+        + "".join(f'printf("d.{f} %zu\\n", offsetof(rt_tensor_desc, {f}));\n' for f, _ in N.RtTensorDesc._fields_)
+        + "".join(f'printf("s.{f} %zu\\n", offsetof(rt_scalars, {f}));\n' for f, _ in N.RtScalars._fields_)
+        + "return 0;}\n")
+    exe = tmp_path / "layout"
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src),
+                           "-o", str(exe)])
+    lines = subprocess.check_output([str(exe)], text=True).split("\n")
+    s_sz, d_sz = map(int, lines[0].split())
+    assert s_sz == ctypes.sizeof(N.RtScalars) and d_sz == ctypes.sizeof(N.RtTensorDesc) == F.DESC_DTYPE.itemsize
+    offs = dict(l.split() for l in lines[1:] if l)
+    for f, _ in N.RtTensorDesc._fields_:
+        assert int(offs["d." + f]) == getattr(N.RtTensorDesc, f).offset == F.DESC_DTYPE.fields[f][1], f
+    for f, _ in N.RtScalars._fields_:
+        assert int(offs["s." + f]) == getattr(N.RtScalars, f).offset, f
+
+
+def test_errors_are_reported_without_a_gpu():
+    L = N.lib()
+    assert L.rt_step_multi(None, None, 0, None, 0, 0, 0, None, None, None) == N.RT_EINVAL
+    assert b"handle" in L.rt_last_error()
+    assert L.rt_sr_copy(None, None, 0, None, 0, None) == N.RT_OK  # empty copy is a no-op
+    assert L.rt_sr_copy(None, None, 8, None, 0, None) == N.RT_EINVAL
+    h = ctypes.c_void_p()
+    rc = L.rt_create(0, ctypes.byref(h))
+    if not torch.cuda.is_available():
+        assert rc != N.RT_OK and L.rt_last_error() != b""
+    with pytest.raises(N.NativeError):
+        N.check(N.RT_EINVAL)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(N, "_lib", None)
+    monkeypatch.setattr(N, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(RuntimeError, match="no fallback"):
+        N.lib()
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "ramtorch_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".h", ".hip")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert not re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M), f
+                assert "liboracle" not in text, f
+
+
+# ---- scalars -----------------------------------------------------------------------------
+@pytest.mark.parametrize("hp,step", [
+    (dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01), 10),
+    (dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01), 1),
+    (dict(lr=2.5e-3, betas=(0.8, 0.9999), eps=1e-10, weight_decay=0.0), 5000),
+])
+def test_make_scalars_agrees_with_oracle_and_known_bits(hp, step):
+    a = F.make_scalars(step=step, **hp)
+    b = oracle.scalars_from_hparams(step=step, **hp)
+    for f in ("beta1", "one_m_beta1", "beta2", "one_m_beta2", "inv_bcs", "eps", "neg_step_size", "apply_decay"):
+        assert getattr(a, f) == getattr(b, f), f
+    if hp["weight_decay"] != 0:
+        assert a.decay == b.decay
+    else:
+        assert a.decay == 1.0 and a.apply_decay == 0
+    if step == 10:
+        bits = lambda x: int(np.float32(x).view(np.uint32))
+        assert bits(a.inv_bcs) == 0x41205C3A and bits(a.neg_step_size) == 0xB920FDF8 and bits(a.decay) == 0x3F7FFFE6
+
+
+# ---- optimizer interface (adamw.py:57-104) -------------------------------------------------
+def _params(dtype=torch.bfloat16):
+    return [torch.nn.Parameter(torch.zeros(4, 6, dtype=dtype)), torch.nn.Parameter(torch.zeros(5, dtype=dtype))]
+
+
+def test_constructor_defaults_and_state_layout():
+    ps = _params()
+    opt = ramtorch_amd.AdamW(ps)
+    g = opt.param_groups[0]
+    assert (g["lr"], g["betas"], g["eps"], g["weight_decay"], g["centralization"]) == (1e-3, (0.9, 0.999), 1e-8, 1e-2, 0)
+    assert opt.chunk_size == 64 and opt.optim_state_dtype == torch.bfloat16 and opt.optim_state_device == "cpu"
+    for p in ps:
+        st = opt.state[p]
+        assert set(st) == {"step", "ema", "ema_squared"}
+        assert st["step"] == 0 and isinstance(st["step"], int)
+        for k in ("ema", "ema_squared"):
+            assert st[k].shape == p.shape and st[k].dtype == torch.bfloat16 and st[k].device.type == "cpu"
+            assert not st[k].any()
+
+
+def test_state_dtype_and_positional_signature():
+    ps = _params(torch.float32)
+    opt = ramtorch_amd.AdamW(ps, 3e-4, (0.95, 0.99), 1e-6, 0.1, 0, 16, torch.float32, "cpu")
+    assert opt.state[ps[0]]["ema"].dtype == torch.float32 and opt.chunk_size == 16
+    assert opt.param_groups[0]["betas"] == (0.95, 0.99)
+
+
+def test_param_groups_from_zero1_style_lists_with_empty_groups():
+    ps = _params()
+    groups = [{"params": [ps[0]], "lr": 1e-3, "weight_decay": 0.01}, {"params": [], "lr": 5e-4, "weight_decay": 0.0},
+              {"params": [ps[1]], "lr": 5e-4}]
+    opt = ramtorch_amd.AdamW(groups)
+    assert [len(g["params"]) for g in opt.param_groups] == [1, 0, 1]
+    assert opt.param_groups[2]["weight_decay"] == 1e-2 and opt.param_groups[1]["lr"] == 5e-4
+    assert opt._tensor_ids() == {id(ps[0]): 0, id(ps[1]): 1}
+
+
+def test_state_dict_round_trip_keeps_reference_keys():
+    ps = _params()
+    opt = ramtorch_amd.AdamW(ps, lr=2e-3)
+    opt.state[ps[0]]["step"] = 7
+    opt.state[ps[0]]["ema"].fill_(0.5)
+    sd = opt.state_dict()
+    assert set(sd) == {"state", "param_groups"}
+    assert set(sd["state"][0]) == {"step", "ema", "ema_squared"}
+    opt2 = ramtorch_amd.AdamW(_params(), lr=1e-3)
+    opt2.load_state_dict(sd)
+    p0 = opt2.param_groups[0]["params"][0]
+    assert opt2.state[p0]["step"] == 7 and opt2.param_groups[0]["lr"] == 2e-3
+    assert torch.equal(opt2.state[p0]["ema"], torch.full((4, 6), 0.5, dtype=torch.bfloat16))
+
+
+def test_step_without_gpu_raises_and_leaves_state_alone():
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    ps = _params()
+    opt = ramtorch_amd.AdamW(ps)
+    ps[0].grad = torch.ones_like(ps[0])
+    with pytest.raises(RuntimeError, match="GPU"):
+        opt.step()
+    assert opt.state[ps[0]]["step"] == 0
+    with pytest.raises(RuntimeError):
+        ramtorch_amd.copy_stochastic_(torch.zeros(4, dtype=torch.bfloat16), torch.zeros(4))
+
+
+def test_zero_grad_and_add_param_group_are_inherited():
+    ps = _params()
+    opt = ramtorch_amd.AdamW([ps[0]])
+    ps[0].grad = torch.ones_like(ps[0])
+    opt.zero_grad()
+    assert ps[0].grad is None
+    opt.add_param_group({"params": [ps[1]], "lr": 1e-5})
+    assert len(opt.param_groups) == 2 and opt.param_groups[1]["betas"] == (0.9, 0.999)
+    assert opt._tensor_ids()[id(ps[1])] == 1
+
+
+# ---- descriptor packing ---------------------------------------------------------------------
+def test_pack_descs_rejects_bad_inputs():
+    t = lambda n, dt=torch.bfloat16: torch.zeros(n, dtype=dt)
+    e = F.Entry(p=t(8), g=t(8), m=t(8), v=t(8), step=1, scalars_idx=0, tensor_id=0)
+    with pytest.raises(ValueError, match="CPU tensor"):
+        F.pack_descs([e], streamed=False)
+    d = F.pack_descs([e], streamed=True)
+    assert d["host_mask"][0] == 15 and d["numel"][0] == 8 and d["p"][0] == e.p.data_ptr()
+    with pytest.raises(ValueError, match="element counts"):
+        F.pack_descs([F.Entry(p=t(8), g=t(9), m=t(8), v=t(8), step=1, scalars_idx=0, tensor_id=0)], streamed=True)
+    with pytest.raises(NotImplementedError):
+        F.pack_descs([F.Entry(p=t(8, torch.float16), g=t(8), m=t(8), v=t(8), step=1, scalars_idx=0, tensor_id=0)],
+                     streamed=True)
+    with pytest.raises(NotImplementedError):
+        F.pack_descs([F.Entry(p=t(8), g=t(8, torch.float64), m=t(8), v=t(8), step=1, scalars_idx=0, tensor_id=0)],
+                     streamed=True)
+    with pytest.raises(ValueError, match="contiguous"):
+        F.pack_descs([F.Entry(p=torch.zeros(4, 4, dtype=torch.bfloat16).t(), g=t(16), m=t(16), v=t(16), step=1,
+                              scalars_idx=0, tensor_id=0)], streamed=True)
+
+
+def test_build_module_knows_its_sources():
+    from ramtorch_amd import build
+    for s in build.SOURCES:
+        assert os.path.exists(os.path.join(build.CSRC, s))
+    assert "--offload-arch=gfx950" in build.HIPCC_FLAGS and "-ffp-contract=off" in build.HIPCC_FLAGS
+    i = build.HIPCC_FLAGS.index("-packed-fp32-ops")
+    assert build.HIPCC_FLAGS[i - 3:i] == ["-Xclang", "-target-feature", "-Xclang"]
