@@ -171,6 +171,9 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=32, help="transformer layers of the Llama-shaped set")
     ap.add_argument("--stream-gb", type=float, default=48.2, help="upper bound on pinned host bytes (streamed)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-calibrate", action="store_true",
+                    help="also launch one plain elementwise kernel that reads 1 GiB and writes 1 GiB, so that "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings can be scaled to bytes")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU; the step needs no exchange between GPUs and a multi-GPU "
@@ -191,7 +194,7 @@ def main() -> int:
     noise = None
     opt_kw = dict(storage_device="cuda", seed=1234)
     bytes_per_elem = 14
-    dtype_label = "bf16 storage, f32 arithmetic"
+    dtype_label = "f32"  # arithmetic type; storage is bf16 (or fp32 for the mixed layout)
     if wl == "llama8b":
         shapes = llama3_8b_shapes(args.layers)
         params, grads = build_resident(shapes, g_dtype=torch.bfloat16, v_dtype=torch.bfloat16, device=dev)
@@ -299,6 +302,14 @@ def main() -> int:
         stream_info["h2d_frac_of_peak"] = stream_info["h2d_GBps"] / stream_info["pinned_h2d_peak_GBps"]
         roofline = {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": None,
                     "traffic": None, "note": "host-link bound; see host_link"}
+
+    if args.pmc_calibrate:
+        x = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        y = torch.empty_like(x)
+        torch.cuda.synchronize()
+        torch.add(x, 1.0, out=y)  # vectorized_elementwise_kernel: 2^30 bytes in, 2^30 bytes out
+        torch.cuda.synchronize()
+        del x, y
 
     out = {
         "metric": METRIC, "value": total / (ms_per_step * 1e-3), "unit": "elements/s", "n_gpus": 1,

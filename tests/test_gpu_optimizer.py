@@ -2,6 +2,8 @@
 against the reference's own op sequence, unbiasedness of the Philox rounding,
 grad-norm clip, centralization, copy_stochastic_.  Run with ``-m gpu``.
 """
+import copy
+
 import numpy as np
 import pytest
 import torch
@@ -20,8 +22,16 @@ def dev16(a, dt=torch.bfloat16):
     return torch.from_numpy(a.view(np.int16).copy()).view(dt).cuda()
 
 
+def nmis(a, b):
+    """Number of elements whose bits differ (keeps assertion messages short)."""
+    a, b = a.detach().cpu().contiguous(), b.detach().cpu().contiguous()
+    assert a.shape == b.shape and a.dtype == b.dtype, (a.shape, b.shape, a.dtype, b.dtype)
+    it = {2: torch.int16, 4: torch.int32}[a.element_size()]
+    return int((a.view(it) != b.view(it)).sum())
+
+
 def bits16(t):
-    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16).ravel()
 
 
 def _make_params(shapes, seed, device="cuda"):
@@ -57,9 +67,9 @@ def test_three_steps_match_the_reference_op_sequence():
             grp = opt.param_groups[0 if i < 2 else 1]
             torch_ops.reference_step_ops(ref_p[i], p.grad, ref_m[i], ref_v[i], lr=grp["lr"], betas=grp["betas"],
                                          eps=grp["eps"], weight_decay=grp["weight_decay"], step=step, noise=noise[p])
-            assert torch.equal(p.detach(), ref_p[i]), f"step {step} param {i}"
-            assert torch.equal(opt.state[p]["ema"], ref_m[i]), f"step {step} ema {i}"
-            assert torch.equal(opt.state[p]["ema_squared"], ref_v[i]), f"step {step} ema_squared {i}"
+            assert nmis(p.detach(), ref_p[i]) == 0, f"step {step} param {i}"
+            assert nmis(opt.state[p]["ema"], ref_m[i]) == 0, f"step {step} ema {i}"
+            assert nmis(opt.state[p]["ema_squared"], ref_v[i]) == 0, f"step {step} ema_squared {i}"
             assert opt.state[p]["step"] == step
 
 
@@ -71,7 +81,7 @@ def test_skipped_and_sparse_gradients():
     opt.step()
     torch.cuda.synchronize()
     assert opt.state[ps[0]]["step"] == 1 and opt.state[ps[1]]["step"] == 0  # adamw.py:114: no grad, no step
-    assert torch.equal(ps[1].detach(), before)
+    assert nmis(ps[1].detach(), before) == 0
     emb = torch.nn.Parameter(torch.zeros(10, 4, device="cuda"))
     emb.grad = torch.sparse_coo_tensor(torch.tensor([[1], [2]]), torch.tensor([1.0]), (10, 4)).cuda()
     with pytest.raises(RuntimeError, match="sparse"):
@@ -103,7 +113,7 @@ def test_state_dict_resume_continues_bit_exactly():
         for p, g in zip(ps, grads):
             p.grad = g
         a.step()
-    sd = a.state_dict()
+    sd = copy.deepcopy(a.state_dict())   # state_dict() hands out the live tensors; a checkpoint would not
     ps2 = [torch.nn.Parameter(p.detach().clone()) for p in ps]
     b = ramtorch_amd.AdamW(ps2, storage_device="cuda", seed=11)
     b.load_state_dict(sd)
@@ -113,8 +123,8 @@ def test_state_dict_resume_continues_bit_exactly():
         opt.step()
     torch.cuda.synchronize()
     for p, q in zip(ps, ps2):
-        assert torch.equal(p.detach(), q.detach())
-        assert torch.equal(a.state[p]["ema_squared"], b.state[q]["ema_squared"]) and b.state[q]["step"] == 3
+        assert nmis(p.detach(), q.detach()) == 0
+        assert nmis(a.state[p]["ema_squared"], b.state[q]["ema_squared"]) == 0 and b.state[q]["step"] == 3
 
 
 def test_non_contiguous_param_round_trips():
@@ -127,7 +137,7 @@ def test_non_contiguous_param_round_trips():
     base.grad, ref.grad = g, g.contiguous()
     o1.step(), o2.step()
     torch.cuda.synchronize()
-    assert torch.equal(base.detach().contiguous(), ref.detach())
+    assert nmis(base.detach().contiguous(), ref.detach()) == 0
 
 
 def test_philox_rounding_is_unbiased_over_1e8_elements():
@@ -196,7 +206,7 @@ def test_grad_norm_clip_and_skip():
     assert np.float32(out[1].item()) == oracle.clip_coef(np.float32(total), 0.01)
     assert out.view(torch.int32)[2].item() == 0
     again = F.grad_norm(h, grads, inv_loss_scale=1 / 1024, max_norm=0.01)
-    assert torch.equal(out[:2], again[:2])  # deterministic reduction order
+    assert nmis(out[:2], again[:2]) == 0  # deterministic reduction order
     grads[2][5] = float("inf")
     bad = F.grad_norm(h, grads, inv_loss_scale=1 / 1024, max_norm=0.01)
     assert bad.view(torch.int32)[2].item() == 1 and float(bad[1]) == 1.0
@@ -230,7 +240,7 @@ def test_optimizer_with_loss_scale_and_max_grad_norm():
     gmap[ps[0]][0, 0] = float("nan")
     opt.step(grads=gmap)
     torch.cuda.synchronize()
-    assert all(torch.equal(a, b.detach()) for a, b in zip(snap, ps))
+    assert all(nmis(a, b.detach()) == 0 for a, b in zip(snap, ps))
     assert opt.last_grad_norm.view(torch.int32)[2].item() == 1
 
 
@@ -272,10 +282,10 @@ def test_copy_stochastic():
     np.testing.assert_array_equal(bits16(tgt), want)
     ref = torch.empty_like(tgt)
     torch_ops.sr_write_(ref, src, torch_ops.noise_to_i32(noise))   # the reference's integer ops on the GPU
-    assert torch.equal(ref, tgt)
+    assert nmis(ref, tgt) == 0
     ramtorch_amd.copy_stochastic_(tgt, src, seed=42)
     torch.cuda.synchronize()
     np.testing.assert_array_equal(bits16(tgt), oracle.sr_copy(src.cpu().numpy(), seed=42))
     cpu_tgt = torch.empty(n, dtype=torch.bfloat16)
     ramtorch_amd.copy_stochastic_(cpu_tgt, src, seed=42)
-    assert torch.equal(cpu_tgt, tgt.cpu())
+    assert nmis(cpu_tgt, tgt.cpu()) == 0

@@ -32,8 +32,16 @@ def dev16(a, dt=torch.bfloat16):
     return torch.from_numpy(a.view(np.int16).copy()).view(dt).cuda()
 
 
+def nmis(a, b):
+    """Number of elements whose bits differ (keeps assertion messages short)."""
+    a, b = a.detach().cpu().contiguous(), b.detach().cpu().contiguous()
+    assert a.shape == b.shape and a.dtype == b.dtype, (a.shape, b.shape, a.dtype, b.dtype)
+    it = {2: torch.int16, 4: torch.int32}[a.element_size()]
+    return int((a.view(it) != b.view(it)).sum())
+
+
 def bits16(t):
-    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16).ravel()
 
 
 def bits32(t):
@@ -287,7 +295,7 @@ def test_elem_offset_pieces_equal_whole(handle):
               for a, b in zip(cuts[:-1], cuts[1:])]
     F.step_resident(handle, pieces, [sc], seed=5, explicit_noise=False)
     torch.cuda.synchronize()
-    assert torch.equal(whole.p, P) and torch.equal(whole.m, M) and torch.equal(whole.v, V)
+    assert nmis(whole.p, P) == 0 and nmis(whole.m, M) == 0 and nmis(whole.v, V) == 0
 
 
 # ---- skip flag ----------------------------------------------------------------------------------------

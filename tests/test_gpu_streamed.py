@@ -24,8 +24,16 @@ def dev16(a):
     return torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16).cuda()
 
 
+def nmis(a, b):
+    """Number of elements whose bits differ (keeps assertion messages short)."""
+    a, b = a.detach().cpu().contiguous(), b.detach().cpu().contiguous()
+    assert a.shape == b.shape and a.dtype == b.dtype, (a.shape, b.shape, a.dtype, b.dtype)
+    it = {2: torch.int16, 4: torch.int32}[a.element_size()]
+    return int((a.view(it) != b.view(it)).sum())
+
+
 def bits16(t):
-    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16).ravel()
 
 
 @pytest.fixture(scope="module")
@@ -97,7 +105,7 @@ def test_streamed_and_resident_agree_bit_for_bit(handle):
     F.step_streamed(handle, [s], [sc], seed=5, explicit_noise=False, chunk_elems=40_000)
     torch.cuda.synchronize()
     for a, b in ((r.p, s.p), (r.m, s.m), (r.v, s.v)):
-        assert torch.equal(a.cpu(), b)
+        assert nmis(a.cpu(), b) == 0
 
 
 def test_optimizer_default_layout_cpu_params_and_pinned_states():
