@@ -111,28 +111,34 @@ static int dtype_size(int dt) { return dt == RT_DT_F32 ? 4 : 2; }
 using MultiKernel = void (*)(const DevTensor*, const ChunkRef*, const DevScalars*, uint32_t, uint32_t,
                              const float*, const uint32_t*);
 
+struct KernelPair {
+    MultiKernel fast;     // chunks wholly inside an aligned tensor
+    MultiKernel generic;  // tails, unaligned tensors, debug outputs, centralization
+};
+
 template <int P, int G, int M, int V>
-static MultiKernel pick_noise(int noise) {
-    return noise == RT_NOISE_EXPLICIT ? sr_adamw_multi_kernel<P, G, M, V, RT_NOISE_EXPLICIT>
-                                      : sr_adamw_multi_kernel<P, G, M, V, RT_NOISE_PHILOX>;
+static KernelPair pick_noise(int noise) {
+    if (noise == RT_NOISE_EXPLICIT)
+        return {sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_EXPLICIT>, sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_EXPLICIT>};
+    return {sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_PHILOX>, sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_PHILOX>};
 }
 template <int P, int G, int M>
-static MultiKernel pick_v(int v, int noise) {
+static KernelPair pick_v(int v, int noise) {
     return v == RT_DT_BF16 ? pick_noise<P, G, M, RT_DT_BF16>(noise) : pick_noise<P, G, M, RT_DT_F32>(noise);
 }
 template <int P, int G>
-static MultiKernel pick_m(int m, int v, int noise) {
+static KernelPair pick_m(int m, int v, int noise) {
     return m == RT_DT_BF16 ? pick_v<P, G, RT_DT_BF16>(v, noise) : pick_v<P, G, RT_DT_F32>(v, noise);
 }
 template <int P>
-static MultiKernel pick_g(int g, int m, int v, int noise) {
+static KernelPair pick_g(int g, int m, int v, int noise) {
     switch (g) {
         case RT_DT_BF16: return pick_m<P, RT_DT_BF16>(m, v, noise);
         case RT_DT_F32: return pick_m<P, RT_DT_F32>(m, v, noise);
         default: return pick_m<P, RT_DT_F16>(m, v, noise);
     }
 }
-static MultiKernel pick_kernel(int p, int g, int m, int v, int noise) {
+static KernelPair pick_kernel(int p, int g, int m, int v, int noise) {
     return p == RT_DT_BF16 ? pick_g<RT_DT_BF16>(g, m, v, noise) : pick_g<RT_DT_F32>(g, m, v, noise);
 }
 
@@ -194,8 +200,8 @@ namespace {
 
 struct Batch {            // tensors of one dtype combination inside a table image
     uint32_t combo;
-    uint32_t first_chunk;
-    uint32_t n_chunks;
+    uint32_t first_fast, n_fast;        // chunk range of the fast kernel
+    uint32_t first_generic, n_generic;  // chunk range of the generic kernel
 };
 
 struct Plan {
@@ -271,14 +277,33 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
     uint8_t* gdt = img + plan.off_gdt;
     uint32_t c = 0;
     plan.batches.clear();
-    for (size_t k = 0; k < order.size(); ++k) {
-        const rt_tensor_desc& d = descs[order[k]];
-        const uint32_t combo = combo_of(d);
-        if (plan.batches.empty() || plan.batches.back().combo != combo) plan.batches.push_back({combo, c, 0});
-        const uint32_t nc = (uint32_t)((d.numel + kChunkElems - 1) / kChunkElems);
-        for (uint32_t j = 0; j < nc; ++j) cr[c++] = ChunkRef{(uint32_t)k, j};
-        plan.batches.back().n_chunks += nc;
-        gdt[k] = d.g_dtype;
+    // Per combination: first every chunk the fast kernel may take (whole chunks of
+    // aligned tensors without debug outputs or centralization), then the rest.
+    size_t k0 = 0;
+    while (k0 < order.size()) {
+        const uint32_t combo = combo_of(descs[order[k0]]);
+        size_t k1 = k0;
+        while (k1 < order.size() && combo_of(descs[order[k1]]) == combo) ++k1;
+        Batch b{combo, c, 0, 0, 0};
+        auto n_whole = [&](size_t k) -> uint32_t {
+            const DevTensor& t = tens[k];
+            const bool plain = (t.flags & kFlagAligned) && (t.dp | t.dm | t.dv | t.row_mean) == 0;
+            return plain ? (uint32_t)(t.numel / kChunkElems) : 0u;
+        };
+        for (size_t k = k0; k < k1; ++k) {
+            const uint32_t nw = n_whole(k);
+            for (uint32_t j = 0; j < nw; ++j) cr[c++] = ChunkRef{(uint32_t)k, j};
+        }
+        b.n_fast = c - b.first_fast;
+        b.first_generic = c;
+        for (size_t k = k0; k < k1; ++k) {
+            const uint32_t nc = (uint32_t)((tens[k].numel + kChunkElems - 1) / kChunkElems);
+            for (uint32_t j = n_whole(k); j < nc; ++j) cr[c++] = ChunkRef{(uint32_t)k, j};
+            gdt[k] = descs[order[k]].g_dtype;
+        }
+        b.n_generic = c - b.first_generic;
+        plan.batches.push_back(b);
+        k0 = k1;
     }
 }
 
@@ -330,11 +355,19 @@ static int launch_update(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, 
     const ChunkRef* chunks = (const ChunkRef*)(base + plan.off_chunks);
     if (h->timing) HIP_TRY(hipEventRecord(h->t0, stream));
     for (const Batch& b : plan.batches) {
-        MultiKernel k = pick_kernel(b.combo & 3, (b.combo >> 2) & 3, (b.combo >> 4) & 3, (b.combo >> 6) & 3,
-                                    noise_mode);
-        hipLaunchKernelGGL(k, dim3(b.n_chunks), dim3(kThreads), 0, stream, tens, chunks + b.first_chunk, sets,
-                           (uint32_t)seed, (uint32_t)(seed >> 32), d_clip_coef, d_skip);
-        HIP_TRY(hipGetLastError());
+        const KernelPair k = pick_kernel(b.combo & 3, (b.combo >> 2) & 3, (b.combo >> 4) & 3, (b.combo >> 6) & 3,
+                                         noise_mode);
+        if (b.n_fast) {
+            hipLaunchKernelGGL(k.fast, dim3(b.n_fast), dim3(kThreads), 0, stream, tens, chunks + b.first_fast, sets,
+                               (uint32_t)seed, (uint32_t)(seed >> 32), d_clip_coef, d_skip);
+            HIP_TRY(hipGetLastError());
+        }
+        if (b.n_generic) {
+            hipLaunchKernelGGL(k.generic, dim3(b.n_generic), dim3(kThreads), 0, stream, tens,
+                               chunks + b.first_generic, sets, (uint32_t)seed, (uint32_t)(seed >> 32), d_clip_coef,
+                               d_skip);
+            HIP_TRY(hipGetLastError());
+        }
     }
     if (h->timing) {
         HIP_TRY(hipEventRecord(h->t1, stream));
