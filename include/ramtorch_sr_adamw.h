@@ -178,10 +178,31 @@ int rt_set_timing(rt_handle* h, int enabled);
 int rt_last_kernel_ms(rt_handle* h, float* ms);
 
 /*
+ * Diagnostic, not in the reference: runs the memory traffic of the all-bf16
+ * update (read p, g, m, v; write p, m, v in place; 14 bytes per element, same
+ * chunking) without the arithmetic, `reps` times after one warm-up, and
+ * returns the mean milliseconds per pass.  14 * numel / time is the rate this
+ * access pattern can reach on the device: the practical ceiling the update
+ * kernel is compared with.  The arrays are bf16-sized scratch of `numel`
+ * elements (a multiple of 8192), 16-byte aligned; p, m, v are overwritten.
+ * Blocks until done.
+ */
+int rt_stream_probe(rt_handle* h, void* p, const void* g, void* m, void* v, uint64_t numel, int reps,
+                    float* ms_out, void* stream);
+
+/*
  * Streamed-path statistics of the most recent rt_step_streamed:
  * out[0] = bytes H2D, out[1] = bytes D2H, out[2] = wall seconds of the call.
  */
 int rt_streamed_stats(rt_handle* h, double out[3]);
+
+/*
+ * Per-chunk timeline of the most recent rt_step_streamed made while timing was
+ * enabled (rt_set_timing): four floats per chunk, milliseconds since the first
+ * H2D began: H2D begin, H2D end, D2H begin, D2H end.  *n_out receives the
+ * number of floats available; at most `cap` are written to `out` (may be NULL).
+ */
+int rt_streamed_timeline(rt_handle* h, float* out, uint32_t cap, uint32_t* n_out);
 
 #ifdef __cplusplus
 }

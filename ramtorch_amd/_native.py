@@ -5,8 +5,11 @@ not load, every entry point raises -- there is no fallback path.
 """
 from __future__ import annotations
 
+import atexit
 import ctypes
 import os
+import sys
+import weakref
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "_lib", "libramtorch_sr_adamw.so")
@@ -23,6 +26,7 @@ RT_HOST_P, RT_HOST_G, RT_HOST_M, RT_HOST_V = 1, 2, 4, 8
 EXPORTS = (
     "rt_version", "rt_last_error", "rt_create", "rt_destroy", "rt_step_multi", "rt_step_streamed",
     "rt_grad_norm", "rt_row_means", "rt_sr_copy", "rt_set_timing", "rt_last_kernel_ms", "rt_streamed_stats",
+    "rt_stream_probe", "rt_streamed_timeline",
 )
 
 
@@ -120,6 +124,10 @@ def lib() -> ctypes.CDLL:
     L.rt_set_timing.argtypes = [vp, i32]
     L.rt_last_kernel_ms.restype = i32
     L.rt_last_kernel_ms.argtypes = [vp, ctypes.POINTER(ctypes.c_float)]
+    L.rt_stream_probe.restype = i32
+    L.rt_stream_probe.argtypes = [vp, vp, vp, vp, vp, u64, i32, ctypes.POINTER(ctypes.c_float), vp]
+    L.rt_streamed_timeline.restype = i32
+    L.rt_streamed_timeline.argtypes = [vp, ctypes.POINTER(ctypes.c_float), u32, ctypes.POINTER(u32)]
     L.rt_streamed_stats.restype = i32
     L.rt_streamed_stats.argtypes = [vp, ctypes.POINTER(ctypes.c_double)]
     v = L.rt_version()
@@ -141,6 +149,7 @@ class Handle:
         self._h = ctypes.c_void_p()
         check(lib().rt_create(int(device), ctypes.byref(self._h)))
         self.device = int(device)
+        _live_handles.add(self)
 
     @property
     def ptr(self) -> ctypes.c_void_p:
@@ -154,6 +163,10 @@ class Handle:
             self._h = ctypes.c_void_p()
 
     def __del__(self):
+        # During interpreter shutdown the HIP runtime may already be gone; the
+        # atexit hook below has released everything that was still open.
+        if sys is None or sys.is_finalizing():
+            return
         try:
             self.close()
         except Exception:
@@ -181,10 +194,37 @@ class Handle:
         check(lib().rt_last_kernel_ms(self.ptr, ctypes.byref(ms)))
         return ms.value
 
+    def stream_probe(self, p, g, m, v, numel, reps=5, stream=0) -> float:
+        """Mean ms per pass of the math-free traffic pattern (see rt_stream_probe)."""
+        ms = ctypes.c_float()
+        check(lib().rt_stream_probe(self.ptr, p, g, m, v, numel, reps, ctypes.byref(ms), stream))
+        return ms.value
+
+    def streamed_timeline(self):
+        """[(h2d_begin, h2d_end, d2h_begin, d2h_end), ...] in ms for the last timed streamed call."""
+        n = ctypes.c_uint32()
+        check(lib().rt_streamed_timeline(self.ptr, None, 0, ctypes.byref(n)))
+        buf = (ctypes.c_float * max(n.value, 1))()
+        check(lib().rt_streamed_timeline(self.ptr, buf, n.value, ctypes.byref(n)))
+        return [tuple(buf[i:i + 4]) for i in range(0, n.value, 4)]
+
     def streamed_stats(self):
         out = (ctypes.c_double * 3)()
         check(lib().rt_streamed_stats(self.ptr, out))
         return {"bytes_h2d": out[0], "bytes_d2h": out[1], "seconds": out[2]}
+
+
+_live_handles: "weakref.WeakSet[Handle]" = weakref.WeakSet()
+
+
+@atexit.register
+def _close_all_handles() -> None:
+    """Release device workspaces while the HIP runtime is still alive."""
+    for h in list(_live_handles):
+        try:
+            h.close()
+        except Exception:
+            pass
 
 
 def sr_copy(target_ptr, source_ptr, numel, noise_ptr, seed, stream=0) -> None:

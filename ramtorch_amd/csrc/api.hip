@@ -68,8 +68,13 @@ struct Streamed {
     hipEvent_t comp_done[2] = {nullptr, nullptr};
     hipEvent_t d2h_done[2] = {nullptr, nullptr};
     DevBuf stage[4][2];  // [p,g,m,v][buffer]
+    DevBuf tables;       // table images of every chunk of the current call, back to back
+    void* tables_host = nullptr;  // pinned image of `tables`
+    size_t tables_host_cap = 0;
     bool ready = false;
     double bytes_h2d = 0, bytes_d2h = 0, seconds = 0;
+    std::vector<hipEvent_t> tl_events;  // 4 per chunk when timing is on: H2D begin/end, D2H begin/end
+    std::vector<float> timeline;        // ms since the first H2D began
 };
 
 }  // namespace
@@ -340,20 +345,12 @@ static int stage_image(rt_handle* h, const Plan& plan, hipStream_t stream, Table
     return RT_OK;
 }
 
-static int launch_update(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
-                         uint64_t seed, int noise_mode, const float* d_clip_coef, const uint32_t* d_skip,
-                         hipStream_t stream) {
-    Plan plan;
-    build_image(h, descs, n, scalars, noise_mode == RT_NOISE_EXPLICIT, plan);
-    if (plan.n_chunks == 0) return RT_OK;
-    TableSlot* slot = nullptr;
-    int rc = stage_image(h, plan, stream, &slot);
-    if (rc != RT_OK) return rc;
-    const uint8_t* base = (const uint8_t*)slot->dev.ptr;
+// Enqueues the update kernels of one table image that already sits in device memory at `base`.
+static int enqueue_kernels(const Plan& plan, const uint8_t* base, uint64_t seed, int noise_mode,
+                           const float* d_clip_coef, const uint32_t* d_skip, hipStream_t stream) {
     const DevScalars* sets = (const DevScalars*)(base + plan.off_sets);
     const DevTensor* tens = (const DevTensor*)(base + plan.off_tensors);
     const ChunkRef* chunks = (const ChunkRef*)(base + plan.off_chunks);
-    if (h->timing) HIP_TRY(hipEventRecord(h->t0, stream));
     for (const Batch& b : plan.batches) {
         const KernelPair k = pick_kernel(b.combo & 3, (b.combo >> 2) & 3, (b.combo >> 4) & 3, (b.combo >> 6) & 3,
                                          noise_mode);
@@ -369,6 +366,21 @@ static int launch_update(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, 
             HIP_TRY(hipGetLastError());
         }
     }
+    return RT_OK;
+}
+
+static int launch_update(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
+                         uint64_t seed, int noise_mode, const float* d_clip_coef, const uint32_t* d_skip,
+                         hipStream_t stream) {
+    Plan plan;
+    build_image(h, descs, n, scalars, noise_mode == RT_NOISE_EXPLICIT, plan);
+    if (plan.n_chunks == 0) return RT_OK;
+    TableSlot* slot = nullptr;
+    int rc = stage_image(h, plan, stream, &slot);
+    if (rc != RT_OK) return rc;
+    if (h->timing) HIP_TRY(hipEventRecord(h->t0, stream));
+    rc = enqueue_kernels(plan, (const uint8_t*)slot->dev.ptr, seed, noise_mode, d_clip_coef, d_skip, stream);
+    if (rc != RT_OK) return rc;
     if (h->timing) {
         HIP_TRY(hipEventRecord(h->t1, stream));
         h->timed = true;
@@ -430,6 +442,9 @@ int rt_destroy(rt_handle* h) {
         if (st.comp_done[b]) (void)hipEventDestroy(st.comp_done[b]);
         if (st.d2h_done[b]) (void)hipEventDestroy(st.d2h_done[b]);
     }
+    if (st.tables.ptr) (void)hipFree(st.tables.ptr);
+    if (st.tables_host) (void)hipHostFree(st.tables_host);
+    for (hipEvent_t e : st.tl_events) (void)hipEventDestroy(e);
     if (st.start) (void)hipEventDestroy(st.start);
     if (st.h2d) (void)hipStreamDestroy(st.h2d);
     if (st.comp) (void)hipStreamDestroy(st.comp);
@@ -668,21 +683,15 @@ int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, cons
                 if (rc != RT_OK) return rc;
             }
 
-    // grads (and anything else already queued by the caller) must be ready
-    HIP_TRY(hipEventRecord(st.start, user));
-    HIP_TRY(hipStreamWaitEvent(st.h2d, st.start, 0));
-    HIP_TRY(hipStreamWaitEvent(st.comp, st.start, 0));
-
-    st.bytes_h2d = st.bytes_d2h = 0;
-    std::vector<rt_tensor_desc> piece;
-    bool used_buf[2] = {false, false};
+    // ---- descriptors of every piece (pointers into staging for host-resident arrays), and the
+    //      table images of all chunks, uploaded in one copy before the pipeline starts
+    std::vector<std::vector<rt_tensor_desc>> pieces(chunks.size());
+    std::vector<Plan> plans(chunks.size());
+    std::vector<size_t> plan_off(chunks.size());
+    std::vector<uint8_t> blob;
     for (size_t c = 0; c < chunks.size(); ++c) {
         const int b = (int)(c & 1);
-        const auto& segs = chunks[c];
-        // H2D: the buffer is free once the D2H of the chunk two back has finished
-        if (used_buf[b]) HIP_TRY(hipStreamWaitEvent(st.h2d, st.d2h_done[b], 0));
-        piece.clear();
-        for (const Segment& s : segs) {
+        for (const Segment& s : chunks[c]) {
             const rt_tensor_desc& d = descs[s.tensor];
             rt_tensor_desc q = d;
             q.numel = s.count;
@@ -692,17 +701,9 @@ int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, cons
                                dtype_size(d.v_dtype)};
             const void* src[4] = {d.p, d.g, d.m, d.v};
             void* dst[4];
-            for (int a = 0; a < 4; ++a) {
-                if (d.host_mask & (1u << a)) {
-                    dst[a] = (uint8_t*)st.stage[a][b].ptr + s.stage_off * es[a];
-                    const size_t bytes = s.count * es[a];
-                    HIP_TRY(hipMemcpyAsync(dst[a], (const uint8_t*)src[a] + s.start * es[a], bytes,
-                                           hipMemcpyHostToDevice, st.h2d));
-                    st.bytes_h2d += (double)bytes;
-                } else {
-                    dst[a] = (uint8_t*)src[a] + s.start * es[a];
-                }
-            }
+            for (int a = 0; a < 4; ++a)
+                dst[a] = (d.host_mask & (1u << a)) ? (void*)((uint8_t*)st.stage[a][b].ptr + s.stage_off * es[a])
+                                                   : (void*)((uint8_t*)src[a] + s.start * es[a]);
             q.p = dst[0]; q.g = dst[1]; q.m = dst[2]; q.v = dst[3];
             if (d.noise_p) q.noise_p = (const uint8_t*)d.noise_p + s.start * 2;
             if (d.noise_m) q.noise_m = (const uint8_t*)d.noise_m + s.start * 2;
@@ -710,25 +711,85 @@ int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, cons
             if (d.dbg_p) q.dbg_p = d.dbg_p + s.start;
             if (d.dbg_m) q.dbg_m = d.dbg_m + s.start;
             if (d.dbg_v) q.dbg_v = d.dbg_v + s.start;
-            piece.push_back(q);
+            pieces[c].push_back(q);
         }
+        build_image(h, pieces[c].data(), (uint32_t)pieces[c].size(), scalars, noise_mode == RT_NOISE_EXPLICIT,
+                    plans[c]);
+        plan_off[c] = align_up(blob.size(), 256);
+        blob.resize(plan_off[c] + plans[c].bytes);
+        if (plans[c].bytes) memcpy(blob.data() + plan_off[c], h->image.data(), plans[c].bytes);
+    }
+    if (blob.size() > st.tables_host_cap) {
+        if (st.tables_host) HIP_TRY(hipHostFree(st.tables_host));
+        st.tables_host = nullptr;
+        st.tables_host_cap = 0;
+        const size_t want = blob.size() + blob.size() / 4 + 4096;
+        hipError_t e = hipHostMalloc(&st.tables_host, want, hipHostMallocDefault);
+        if (e != hipSuccess) return fail(RT_ENOMEM, "hipHostMalloc(%zu) failed: %s", want, hipGetErrorString(e));
+        st.tables_host_cap = want;
+    }
+    rc = dev_reserve(st.tables, blob.size());
+    if (rc != RT_OK) return rc;
+    memcpy(st.tables_host, blob.data(), blob.size());
+
+    // grads (and anything else already queued by the caller) must be ready
+    HIP_TRY(hipEventRecord(st.start, user));
+    HIP_TRY(hipStreamWaitEvent(st.h2d, st.start, 0));
+    HIP_TRY(hipStreamWaitEvent(st.comp, st.start, 0));
+    if (!blob.empty())
+        HIP_TRY(hipMemcpyAsync(st.tables.ptr, st.tables_host, blob.size(), hipMemcpyHostToDevice, st.comp));
+
+    st.bytes_h2d = st.bytes_d2h = 0;
+    st.timeline.clear();
+    const bool trace = h->timing;
+    if (trace) {
+        while (st.tl_events.size() < 4 * chunks.size()) {
+            hipEvent_t e;
+            HIP_TRY(hipEventCreate(&e));
+            st.tl_events.push_back(e);
+        }
+    }
+    bool used_buf[2] = {false, false};
+    for (size_t c = 0; c < chunks.size(); ++c) {
+        const int b = (int)(c & 1);
+        const auto& segs = chunks[c];
+        // H2D: the buffer is free once the D2H of the chunk two back has finished
+        if (used_buf[b]) HIP_TRY(hipStreamWaitEvent(st.h2d, st.d2h_done[b], 0));
+        if (trace) HIP_TRY(hipEventRecord(st.tl_events[4 * c + 0], st.h2d));
+        for (size_t k = 0; k < segs.size(); ++k) {
+            const Segment& s = segs[k];
+            const rt_tensor_desc& d = descs[s.tensor];
+            const int es[4] = {dtype_size(d.p_dtype), dtype_size(d.g_dtype), dtype_size(d.m_dtype),
+                               dtype_size(d.v_dtype)};
+            const void* host[4] = {d.p, d.g, d.m, d.v};
+            void* dev[4] = {pieces[c][k].p, (void*)pieces[c][k].g, pieces[c][k].m, pieces[c][k].v};
+            for (int a = 0; a < 4; ++a) {
+                if (!(d.host_mask & (1u << a))) continue;
+                const size_t bytes = s.count * es[a];
+                HIP_TRY(hipMemcpyAsync(dev[a], (const uint8_t*)host[a] + s.start * es[a], bytes,
+                                       hipMemcpyHostToDevice, st.h2d));
+                st.bytes_h2d += (double)bytes;
+            }
+        }
+        if (trace) HIP_TRY(hipEventRecord(st.tl_events[4 * c + 1], st.h2d));
         HIP_TRY(hipEventRecord(st.h2d_done[b], st.h2d));
 
         // compute
         HIP_TRY(hipStreamWaitEvent(st.comp, st.h2d_done[b], 0));
-        rc = launch_update(h, piece.data(), (uint32_t)piece.size(), scalars, seed, noise_mode, nullptr, nullptr,
-                           st.comp);
+        rc = enqueue_kernels(plans[c], (const uint8_t*)st.tables.ptr + plan_off[c], seed, noise_mode, nullptr,
+                             nullptr, st.comp);
         if (rc != RT_OK) return rc;
         HIP_TRY(hipEventRecord(st.comp_done[b], st.comp));
 
         // D2H of the updated host-resident arrays (p, m, v; grads are read-only)
         HIP_TRY(hipStreamWaitEvent(st.d2h, st.comp_done[b], 0));
+        if (trace) HIP_TRY(hipEventRecord(st.tl_events[4 * c + 2], st.d2h));
         for (size_t k = 0; k < segs.size(); ++k) {
             const Segment& s = segs[k];
             const rt_tensor_desc& d = descs[s.tensor];
             const int es[4] = {dtype_size(d.p_dtype), 0, dtype_size(d.m_dtype), dtype_size(d.v_dtype)};
             void* host[4] = {d.p, nullptr, d.m, d.v};
-            const void* dev[4] = {piece[k].p, nullptr, piece[k].m, piece[k].v};
+            const void* dev[4] = {pieces[c][k].p, nullptr, pieces[c][k].m, pieces[c][k].v};
             for (int a = 0; a < 4; ++a) {
                 if (a == 1 || !(d.host_mask & (1u << a))) continue;
                 const size_t bytes = s.count * es[a];
@@ -737,6 +798,7 @@ int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, cons
                 st.bytes_d2h += (double)bytes;
             }
         }
+        if (trace) HIP_TRY(hipEventRecord(st.tl_events[4 * c + 3], st.d2h));
         HIP_TRY(hipEventRecord(st.d2h_done[b], st.d2h));
         used_buf[b] = true;
     }
@@ -744,6 +806,49 @@ int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, cons
     HIP_TRY(hipStreamSynchronize(st.d2h));
     HIP_TRY(hipStreamSynchronize(st.comp));
     st.seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - wall0).count();
+    if (trace) {
+        st.timeline.resize(4 * chunks.size());
+        for (size_t i = 0; i < st.timeline.size(); ++i)
+            HIP_TRY(hipEventElapsedTime(&st.timeline[i], st.tl_events[0], st.tl_events[i]));
+    }
+    return RT_OK;
+}
+
+int rt_streamed_timeline(rt_handle* h, float* out, uint32_t cap, uint32_t* n_out) {
+    if (!h || !n_out) return fail(RT_EINVAL, "NULL argument");
+    const uint32_t n = (uint32_t)h->st.timeline.size();
+    *n_out = n;
+    if (out)
+        for (uint32_t i = 0; i < n && i < cap; ++i) out[i] = h->st.timeline[i];
+    return RT_OK;
+}
+
+int rt_stream_probe(rt_handle* h, void* p, const void* g, void* m, void* v, uint64_t numel, int reps, float* ms_out,
+                    void* stream_) {
+    if (!h || !ms_out) return fail(RT_EINVAL, "NULL argument");
+    if (!p || !g || !m || !v) return fail(RT_EINVAL, "NULL array pointer");
+    if ((((uintptr_t)p | (uintptr_t)g | (uintptr_t)m | (uintptr_t)v) & 15u) != 0)
+        return fail(RT_EINVAL, "arrays must be 16-byte aligned");
+    if (numel == 0 || numel % kChunkElems != 0 || numel / kChunkElems > 0x7FFFFFFFull)
+        return fail(RT_EINVAL, "numel must be a positive multiple of %u", kChunkElems);
+    if (reps < 1) return fail(RT_EINVAL, "reps must be >= 1");
+    hipStream_t stream = (hipStream_t)stream_;
+    HIP_TRY(hipSetDevice(h->device));
+    const dim3 grid((uint32_t)(numel / kChunkElems));
+    hipLaunchKernelGGL(stream_probe_kernel, grid, dim3(kThreads), 0, stream, (uint64_t)p, (uint64_t)g, (uint64_t)m,
+                       (uint64_t)v);  // warm-up (page tables, clocks)
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipEventRecord(h->t0, stream));
+    for (int r = 0; r < reps; ++r)
+        hipLaunchKernelGGL(stream_probe_kernel, grid, dim3(kThreads), 0, stream, (uint64_t)p, (uint64_t)g,
+                           (uint64_t)m, (uint64_t)v);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipEventRecord(h->t1, stream));
+    HIP_TRY(hipEventSynchronize(h->t1));
+    float ms = 0.0f;
+    HIP_TRY(hipEventElapsedTime(&ms, h->t0, h->t1));
+    *ms_out = ms / (float)reps;
+    h->timed = false;
     return RT_OK;
 }
 

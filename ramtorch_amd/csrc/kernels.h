@@ -412,6 +412,31 @@ __global__ __launch_bounds__(kThreads) void sr_adamw_generic_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// Stream probe: the memory traffic of the all-bf16 fast kernel (read p, g, m, v;
+// write p, m, v in place, same chunking and prefetch) with the arithmetic
+// replaced by two integer ops.  Its rate is what this access pattern can get
+// out of HBM on the device at hand, i.e. the practical ceiling of the update.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void stream_probe_kernel(uint64_t p, uint64_t g, uint64_t m, uint64_t v) {
+    const uint64_t i0 = ((uint64_t)blockIdx.x * kChunkElems + (uint64_t)threadIdx.x * kVec) * 2;
+    constexpr uint64_t kStride = (uint64_t)kThreads * kVec * 2;
+    u32x4 a = ldg128(p + i0), b = ldg128(g + i0), c = ldg128(m + i0), d = ldg128(v + i0);
+#pragma unroll
+    for (int it = 0; it < kItersPerChunk; ++it) {
+        const uint64_t i = i0 + it * kStride;
+        u32x4 na, nb, nc, nd;
+        if (it + 1 < kItersPerChunk) {
+            na = ldg128(p + i + kStride); nb = ldg128(g + i + kStride);
+            nc = ldg128(m + i + kStride); nd = ldg128(v + i + kStride);
+        }
+        stg128(p + i, a ^ b);
+        stg128(m + i, c ^ b);
+        stg128(v + i, d ^ b);
+        if (it + 1 < kItersPerChunk) { a = na; b = nb; c = nc; d = nd; }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // copy_stochastic_ on its own: fp32 -> bf16.  Philox counter word 2 is 3
 // ("which" values 0..2 belong to the step), word 3 is 0.
 // ---------------------------------------------------------------------------
