@@ -145,6 +145,23 @@ def _descs_ptr(d: np.ndarray):
     return d.ctypes.data_as(ctypes.POINTER(N.RtTensorDesc))
 
 
+def launch_resident(handle: N.Handle, descs: np.ndarray, scalars: Sequence[N.RtScalars], *, seed: int,
+                    explicit_noise: bool, clip_coef: Optional[torch.Tensor] = None,
+                    skip: Optional[torch.Tensor] = None, stream: Optional[int] = None) -> None:
+    """``rt_step_multi`` over an already packed ``rt_tensor_desc`` array (every
+    pointer a device address).  Enqueues on ``stream`` (default: torch's current
+    stream) and returns without synchronising; the caller keeps the tensors alive."""
+    if len(descs) == 0:
+        return
+    descs = np.ascontiguousarray(descs)
+    if stream is None:
+        stream = torch.cuda.current_stream(handle.device).cuda_stream
+    handle.step_multi(_descs_ptr(descs), len(descs), scalars_array(scalars), len(scalars), seed & (2 ** 64 - 1),
+                      N.RT_NOISE_EXPLICIT if explicit_noise else N.RT_NOISE_PHILOX,
+                      None if clip_coef is None else clip_coef.data_ptr(),
+                      None if skip is None else skip.data_ptr(), stream)
+
+
 def step_resident(handle: N.Handle, entries: Sequence[Entry], scalars: Sequence[N.RtScalars], *, seed: int,
                   explicit_noise: bool, clip_coef: Optional[torch.Tensor] = None,
                   skip: Optional[torch.Tensor] = None, stream: Optional[int] = None) -> None:
@@ -152,13 +169,8 @@ def step_resident(handle: N.Handle, entries: Sequence[Entry], scalars: Sequence[
     (default: torch's current stream).  Returns without synchronising."""
     if not entries:
         return
-    d = pack_descs(entries, streamed=False)
-    if stream is None:
-        stream = torch.cuda.current_stream(handle.device).cuda_stream
-    handle.step_multi(_descs_ptr(d), len(entries), scalars_array(scalars), len(scalars), seed & (2 ** 64 - 1),
-                      N.RT_NOISE_EXPLICIT if explicit_noise else N.RT_NOISE_PHILOX,
-                      None if clip_coef is None else clip_coef.data_ptr(),
-                      None if skip is None else skip.data_ptr(), stream)
+    launch_resident(handle, pack_descs(entries, streamed=False), scalars, seed=seed, explicit_noise=explicit_noise,
+                    clip_coef=clip_coef, skip=skip, stream=stream)
 
 
 def step_streamed(handle: N.Handle, entries: Sequence[Entry], scalars: Sequence[N.RtScalars], *, seed: int,

@@ -11,6 +11,7 @@ from __future__ import annotations
 
 from typing import Dict, List, Optional
 
+import numpy as np
 import torch
 from torch.optim import Optimizer
 
@@ -25,6 +26,11 @@ def _handle(device_index: int) -> N.Handle:
     if h is None:
         h = _handles[device_index] = N.Handle(device_index)
     return h
+
+
+class _Rec:
+    """Static facts about one parameter and its two states (see AdamW._make_rec)."""
+    __slots__ = ("p", "state", "m", "v", "p_ptr", "m_ptr", "v_ptr", "numel", "tensor_id", "dev", "plain", "codes")
 
 
 def _compute_device_index(p: torch.Tensor) -> int:
@@ -110,6 +116,12 @@ class AdamW(Optimizer):
                 if not self.state[p]:
                     self._init_state(p)
 
+    def __setstate__(self, state):
+        # load_state_dict (and unpickling) replace self.state wholesale: drop everything derived from it
+        super().__setstate__(state)
+        self._recs = None
+        self._desc_cache = {}
+
     # -- state ---------------------------------------------------------------------
     def _new_state_tensor(self, p: torch.Tensor) -> torch.Tensor:
         t = torch.zeros_like(p.data, dtype=self.optim_state_dtype, device=self.optim_state_device,
@@ -134,6 +146,46 @@ class AdamW(Optimizer):
                 k += 1
         return ids
 
+    # -- per-parameter records -----------------------------------------------------------
+    # What the step needs to know about a parameter and its states does not change from
+    # step to step (addresses, sizes, dtypes), so it is gathered once and re-validated
+    # cheaply: the state tensors must be the same objects and the parameter's address the same.
+    def _make_rec(self, p: torch.Tensor, tensor_id: int) -> "_Rec":
+        state = self.state[p]
+        if not state:
+            self._init_state(p)  # adamw.py:125-148
+        m, v = state["ema"], state["ema_squared"]
+        r = _Rec()
+        r.p, r.state, r.m, r.v, r.tensor_id = p, state, m, v, tensor_id
+        r.p_ptr, r.m_ptr, r.v_ptr, r.numel = p.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel()
+        r.dev = _compute_device_index(p)
+        ok_dt = (torch.bfloat16, torch.float32)
+        r.plain = (p.is_cuda and m.is_cuda and v.is_cuda and m.device == p.device and v.device == p.device
+                   and p.is_contiguous() and m.is_contiguous() and v.is_contiguous()
+                   and p.dtype in ok_dt and m.dtype in ok_dt and v.dtype in ok_dt
+                   and m.numel() == r.numel and v.numel() == r.numel)
+        if r.plain:
+            r.codes = (F.dtype_code(p.dtype, "param"), F.dtype_code(m.dtype, "state"), F.dtype_code(v.dtype, "state"))
+        return r
+
+    def _records(self) -> List[List["_Rec"]]:
+        recs = getattr(self, "_recs", None)
+        groups = self.param_groups
+        if recs is not None and len(recs) == len(groups) and all(
+                len(rg) == len(g["params"]) for rg, g in zip(recs, groups)):
+            return recs
+        k = 0
+        recs = []
+        for g in groups:
+            row = []
+            for p in g["params"]:
+                row.append(self._make_rec(p, k))
+                k += 1
+            recs.append(row)
+        self._recs = recs
+        self._desc_cache = {}
+        return recs
+
     # -- step ----------------------------------------------------------------------
     def step(self, closure=None, *, noise=None, debug_out=None, grads=None):
         """One optimizer step (adamw.py:106-234).
@@ -155,42 +207,65 @@ class AdamW(Optimizer):
         if not torch.cuda.is_available():
             raise RuntimeError("ramtorch_amd.AdamW.step needs a GPU: the update runs only as HIP kernels")
 
-        ids = self._tensor_ids()
+        recs = self._records()
         scalars: List[N.RtScalars] = []
         scalar_key: Dict[tuple, int] = {}
+        # plain lane: tensors wholly on one GPU, contiguous, nothing special -> columns only
+        plain: Dict[int, tuple] = {}      # dev -> (recs, grads, grad ptrs, grad codes, steps, scalar idx)
+        # general lane: everything else goes through Entry objects
         resident: Dict[int, List[F.Entry]] = {}
         streamed: Dict[int, List[F.Entry]] = {}
         writeback = []  # (destination, contiguous temporary) pairs for non-contiguous p / states
         inv_loss_scale = 1.0 / self.loss_scale if self.loss_scale != 1.0 else 1.0
+        extras = noise is not None or debug_out is not None
+        dt_code = F._DT_CODE
 
         with torch.no_grad():
             for gi, group in enumerate(self.param_groups):
                 beta1, beta2 = group["betas"]
-                for p in group["params"]:
+                lr, eps, wd, cen = group["lr"], group["eps"], group["weight_decay"], group["centralization"]
+                row = recs[gi]
+                last_step, last_si = None, -1
+                for k, p in enumerate(group["params"]):
                     grad = grads.get(p, p.grad) if grads is not None else p.grad
                     if grad is None:
                         continue  # adamw.py:114: skipped, and its step count does not advance
                     if grad.is_sparse:
                         raise RuntimeError("AdamW does not support sparse gradients")  # adamw.py:118-119
-                    state = self.state[p]
-                    if not state:
-                        self._init_state(p)  # adamw.py:125-148
-                    dev = _compute_device_index(p)
-                    state["step"] += 1  # adamw.py:177
-                    step = state["step"]
-                    key = (gi, step, group["lr"], beta1, beta2, group["eps"], group["weight_decay"],
-                           group["centralization"])
-                    si = scalar_key.get(key)
-                    if si is None:
-                        si = scalar_key[key] = len(scalars)
-                        scalars.append(F.make_scalars(group["lr"], (beta1, beta2), group["eps"],
-                                                      group["weight_decay"], step,
-                                                      centralization=group["centralization"],
-                                                      inv_loss_scale=inv_loss_scale))
-                    keep = []
-                    pt, mt, vt = p.data, state["ema"], state["ema_squared"]
+                    r = row[k]
+                    state = r.state
+                    if (r.p is not p or state.get("ema") is not r.m or state.get("ema_squared") is not r.v
+                            or p.data_ptr() != r.p_ptr or r.m.data_ptr() != r.m_ptr or r.v.data_ptr() != r.v_ptr):
+                        r = row[k] = self._make_rec(p, r.tensor_id)
+                        state = r.state
+                    step = state["step"] + 1  # adamw.py:177
+                    state["step"] = step
+                    if step != last_step:
+                        key = (gi, step, lr, beta1, beta2, eps, wd, cen)
+                        si = scalar_key.get(key)
+                        if si is None:
+                            si = scalar_key[key] = len(scalars)
+                            scalars.append(F.make_scalars(lr, (beta1, beta2), eps, wd, step, centralization=cen,
+                                                          inv_loss_scale=inv_loss_scale))
+                        last_step, last_si = step, si
+                    si = last_si
+                    dev = r.dev
+
+                    gcode = dt_code.get(grad.dtype)
+                    if (r.plain and cen == 0 and gcode is not None and grad.is_cuda and grad.is_contiguous()
+                            and grad.device.index == dev and grad.numel() == r.numel
+                            and not (extras and ((noise is not None and p in noise)
+                                                 or (debug_out is not None and p in debug_out)))):
+                        lane = plain.get(dev)
+                        if lane is None:
+                            lane = plain[dev] = ([], [], [], [], [], [])
+                        lane[0].append(r); lane[1].append(grad); lane[2].append(grad.data_ptr())
+                        lane[3].append(gcode); lane[4].append(step); lane[5].append(si)
+                        continue
+
+                    # ---- general lane ----
                     arrays = []
-                    for t in (pt, mt, vt):
+                    for t in (p.data, r.m, r.v):
                         if t.is_cuda and t.device.index != dev:
                             raise RuntimeError("param and optimizer states live on different GPUs")
                         if not t.is_contiguous():
@@ -206,8 +281,8 @@ class AdamW(Optimizer):
                     if g.dtype not in (torch.bfloat16, torch.float32, torch.float16):
                         g = g.to(torch.float32)  # adamw.py:167 upcasts every gradient to fp32
                     e = F.Entry(p=arrays[0], g=g, m=arrays[1], v=arrays[2], step=step, scalars_idx=si,
-                                tensor_id=ids[id(p)], keep=keep)
-                    if group["centralization"] != 0:
+                                tensor_id=r.tensor_id)
+                    if cen != 0:
                         if self.max_grad_norm is not None:
                             raise NotImplementedError("centralization together with max_grad_norm")
                         if not g.is_cuda:
@@ -228,25 +303,26 @@ class AdamW(Optimizer):
                     (resident if on_gpu else streamed).setdefault(dev, []).append(e)
 
             explicit = noise is not None
-            for dev in sorted(set(resident) | set(streamed)):
+            for dev in sorted(set(plain) | set(resident) | set(streamed)):
                 h = _handle(dev)
                 with torch.cuda.device(dev):
                     res, stm = resident.get(dev, []), streamed.get(dev, [])
+                    lane = plain.get(dev)
+                    descs = self._plain_descs(dev, lane) if lane is not None else None
+                    if res:
+                        d2 = F.pack_descs(res, streamed=False)
+                        descs = d2 if descs is None else np.concatenate([descs, d2])
                     clip = skip = None
                     if self.max_grad_norm is not None:
                         if stm:
                             raise NotImplementedError("max_grad_norm with host-resident params or states")
-                        grads = [e.g for e in res + stm]
-                        for i, g in enumerate(grads):
-                            if not g.is_cuda:
-                                grads[i] = g.to(f"cuda:{dev}", non_blocking=True)
-                        for e, g in zip(res + stm, grads):
-                            e.g = g
-                        out = F.grad_norm(h, grads, inv_loss_scale=inv_loss_scale, max_norm=self.max_grad_norm)
+                        gl = (lane[1] if lane is not None else []) + [e.g for e in res]
+                        out = F.grad_norm(h, gl, inv_loss_scale=inv_loss_scale, max_norm=self.max_grad_norm)
                         self.last_grad_norm = out
                         clip, skip = out[1:2], out[2:3]
-                    F.step_resident(h, res, scalars, seed=self.seed, explicit_noise=explicit, clip_coef=clip,
-                                    skip=skip)
+                    if descs is not None:
+                        F.launch_resident(h, descs, scalars, seed=self.seed, explicit_noise=explicit, clip_coef=clip,
+                                          skip=skip)
                     if stm:
                         chunk_elems = max(8, (self.stream_chunk_bytes // 2) // 8 * 8)
                         F.step_streamed(h, stm, scalars, seed=self.seed, explicit_noise=explicit,
@@ -254,3 +330,28 @@ class AdamW(Optimizer):
             for dst, tmp in writeback:
                 dst.copy_(tmp)
         return loss
+
+    def _plain_descs(self, dev: int, lane) -> np.ndarray:
+        """Descriptor array of the plain lane.  The columns that describe p / m / v are
+        reused from the previous step when the same records step again."""
+        lrecs, _, gptrs, gcodes, steps, sis = lane
+        key = tuple(map(id, lrecs))
+        cached = self._desc_cache.get(dev)
+        if cached is not None and cached[0] == key:
+            d = cached[1]
+        else:
+            d = np.zeros(len(lrecs), F.DESC_DTYPE)
+            d["p"] = [r.p_ptr for r in lrecs]
+            d["m"] = [r.m_ptr for r in lrecs]
+            d["v"] = [r.v_ptr for r in lrecs]
+            d["numel"] = [r.numel for r in lrecs]
+            d["tensor_id"] = [r.tensor_id for r in lrecs]
+            d["p_dtype"] = [r.codes[0] for r in lrecs]
+            d["m_dtype"] = [r.codes[1] for r in lrecs]
+            d["v_dtype"] = [r.codes[2] for r in lrecs]
+            self._desc_cache[dev] = (key, d, lrecs)  # lrecs keeps the ids in `key` alive
+        d["g"] = gptrs
+        d["g_dtype"] = gcodes
+        d["step"] = np.asarray(steps, dtype=np.uint64) & 0xFFFFFFFF
+        d["scalars_idx"] = sis
+        return d
