@@ -142,6 +142,35 @@ int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, cons
                      void* stream);
 
 /*
+ * rt_step_streamed without the final wait, for callers that update one tensor
+ * at a time while other GPU work is still being queued (for instance from the
+ * post-accumulate-grad hook that ramtorch/modules/linear.py:97-111 invokes
+ * inside backward, instead of the D2H + H2D round trip of the gradient in
+ * linear.py:416-427 / adamw.py:167).  Returns as soon as everything is
+ * enqueued; *ticket (optional) identifies the call.  Until the ticket has
+ * completed the caller must keep every array of the call alive and must not
+ * touch p / m / v.  Calls on one handle run in order and share the staging
+ * buffers, so consecutive calls overlap like the chunks of one call.
+ *   rt_streamed_completed: highest ticket whose copies have all landed (non-blocking)
+ *   rt_streamed_wait:      blocks until everything enqueued so far has finished
+ */
+int rt_step_streamed_async(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
+                           uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems,
+                           void* stream, uint64_t* ticket);
+int rt_streamed_wait(rt_handle* h);
+int rt_streamed_completed(rt_handle* h, uint64_t* ticket_done);
+
+/*
+ * The chunk schedule rt_step_streamed would use, without touching a GPU: one
+ * row of five uint64 per piece: chunk index, tensor index, first element inside
+ * the tensor, element count, element offset inside the staging buffers.
+ * *n_out receives the number of pieces; at most `cap` rows are written to
+ * `out` (may be NULL).  Uses only numel of each desc.
+ */
+int rt_streamed_plan(const rt_tensor_desc* descs, uint32_t n, uint64_t chunk_elems, uint64_t* out, uint32_t cap,
+                     uint32_t* n_out);
+
+/*
  * Global gradient norm over n device tensors (uses g, g_dtype, numel of each
  * desc), for the optional clip / skip check; not in the reference.  Writes to
  * d_out (device, 16-byte aligned):

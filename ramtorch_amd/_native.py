@@ -26,7 +26,8 @@ RT_HOST_P, RT_HOST_G, RT_HOST_M, RT_HOST_V = 1, 2, 4, 8
 EXPORTS = (
     "rt_version", "rt_last_error", "rt_create", "rt_destroy", "rt_step_multi", "rt_step_streamed",
     "rt_grad_norm", "rt_row_means", "rt_sr_copy", "rt_set_timing", "rt_last_kernel_ms", "rt_streamed_stats",
-    "rt_stream_probe", "rt_streamed_timeline",
+    "rt_stream_probe", "rt_streamed_timeline", "rt_streamed_plan",
+    "rt_step_streamed_async", "rt_streamed_wait", "rt_streamed_completed",
 )
 
 
@@ -128,6 +129,14 @@ def lib() -> ctypes.CDLL:
     L.rt_stream_probe.argtypes = [vp, vp, vp, vp, vp, u64, i32, ctypes.POINTER(ctypes.c_float), vp]
     L.rt_streamed_timeline.restype = i32
     L.rt_streamed_timeline.argtypes = [vp, ctypes.POINTER(ctypes.c_float), u32, ctypes.POINTER(u32)]
+    L.rt_step_streamed_async.restype = i32
+    L.rt_step_streamed_async.argtypes = [vp, descs, u32, scal, u32, u64, i32, u64, vp, ctypes.POINTER(u64)]
+    L.rt_streamed_wait.restype = i32
+    L.rt_streamed_wait.argtypes = [vp]
+    L.rt_streamed_completed.restype = i32
+    L.rt_streamed_completed.argtypes = [vp, ctypes.POINTER(u64)]
+    L.rt_streamed_plan.restype = i32
+    L.rt_streamed_plan.argtypes = [descs, u32, u64, ctypes.POINTER(u64), u32, ctypes.POINTER(u32)]
     L.rt_streamed_stats.restype = i32
     L.rt_streamed_stats.argtypes = [vp, ctypes.POINTER(ctypes.c_double)]
     v = L.rt_version()
@@ -180,6 +189,21 @@ class Handle:
     def step_streamed(self, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, stream=0):
         check(lib().rt_step_streamed(self.ptr, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, stream))
 
+    def step_streamed_async(self, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, stream=0) -> int:
+        """Enqueue only; returns the ticket of the call."""
+        t = ctypes.c_uint64()
+        check(lib().rt_step_streamed_async(self.ptr, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems,
+                                           stream, ctypes.byref(t)))
+        return t.value
+
+    def streamed_wait(self) -> None:
+        check(lib().rt_streamed_wait(self.ptr))
+
+    def streamed_completed(self) -> int:
+        t = ctypes.c_uint64()
+        check(lib().rt_streamed_completed(self.ptr, ctypes.byref(t)))
+        return t.value
+
     def grad_norm(self, descs, n, inv_loss_scale, max_norm, d_out, stream=0):
         check(lib().rt_grad_norm(self.ptr, descs, n, inv_loss_scale, max_norm, d_out, stream))
 
@@ -225,6 +249,15 @@ def _close_all_handles() -> None:
             h.close()
         except Exception:
             pass
+
+
+def streamed_plan(descs, n: int, chunk_elems: int):
+    """[(chunk, tensor, start, count, stage_offset), ...]: the schedule of rt_step_streamed (host only)."""
+    k = ctypes.c_uint32()
+    check(lib().rt_streamed_plan(descs, n, chunk_elems, None, 0, ctypes.byref(k)))
+    buf = (ctypes.c_uint64 * max(5 * k.value, 1))()
+    check(lib().rt_streamed_plan(descs, n, chunk_elems, buf, k.value, ctypes.byref(k)))
+    return [tuple(buf[5 * i:5 * i + 5]) for i in range(k.value)]
 
 
 def sr_copy(target_ptr, source_ptr, numel, noise_ptr, seed, stream=0) -> None:

@@ -8,6 +8,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <deque>
 #include <map>
 #include <new>
 #include <vector>
@@ -68,9 +69,23 @@ struct Streamed {
     hipEvent_t comp_done[2] = {nullptr, nullptr};
     hipEvent_t d2h_done[2] = {nullptr, nullptr};
     DevBuf stage[4][2];  // [p,g,m,v][buffer]
-    DevBuf tables;       // table images of every chunk of the current call, back to back
-    void* tables_host = nullptr;  // pinned image of `tables`
-    size_t tables_host_cap = 0;
+    // Table images of every chunk of one call, back to back.  A small ring, because an
+    // asynchronous call may still be running when the next one builds its tables.
+    struct TableRing {
+        DevBuf dev;
+        void* host = nullptr;  // pinned image
+        size_t host_cap = 0;
+        hipEvent_t done = nullptr;  // recorded after the last kernel that reads `dev`
+        bool in_flight = false;
+    } ring[4];
+    uint32_t ring_pos = 0;
+    // The pipeline state survives across calls so that asynchronous calls chain correctly:
+    uint64_t seq = 0;                      // chunks enqueued so far; chunk `seq` uses buffer seq & 1
+    bool used_buf[2] = {false, false};     // buffer has a D2H whose completion the next H2D must await
+    bool pending = false;                  // work enqueued since the last wait
+    uint64_t tickets_issued = 0, tickets_done = 0;
+    std::deque<std::pair<uint64_t, hipEvent_t>> ticket_events;  // (ticket, recorded on d2h after its last copy)
+    std::vector<hipEvent_t> event_pool;
     bool ready = false;
     double bytes_h2d = 0, bytes_d2h = 0, seconds = 0;
     std::vector<hipEvent_t> tl_events;  // 4 per chunk when timing is on: H2D begin/end, D2H begin/end
@@ -442,8 +457,13 @@ int rt_destroy(rt_handle* h) {
         if (st.comp_done[b]) (void)hipEventDestroy(st.comp_done[b]);
         if (st.d2h_done[b]) (void)hipEventDestroy(st.d2h_done[b]);
     }
-    if (st.tables.ptr) (void)hipFree(st.tables.ptr);
-    if (st.tables_host) (void)hipHostFree(st.tables_host);
+    for (auto& r : st.ring) {
+        if (r.dev.ptr) (void)hipFree(r.dev.ptr);
+        if (r.host) (void)hipHostFree(r.host);
+        if (r.done) (void)hipEventDestroy(r.done);
+    }
+    for (auto& te : st.ticket_events) (void)hipEventDestroy(te.second);
+    for (hipEvent_t e : st.event_pool) (void)hipEventDestroy(e);
     for (hipEvent_t e : st.tl_events) (void)hipEventDestroy(e);
     if (st.start) (void)hipEventDestroy(st.start);
     if (st.h2d) (void)hipStreamDestroy(st.h2d);
@@ -606,6 +626,7 @@ static int streamed_init(rt_handle* h) {
         HIP_TRY(hipEventCreateWithFlags(&st.comp_done[b], hipEventDisableTiming));
         HIP_TRY(hipEventCreateWithFlags(&st.d2h_done[b], hipEventDisableTiming));
     }
+    for (auto& r : st.ring) HIP_TRY(hipEventCreateWithFlags(&r.done, hipEventDisableTiming));
     st.ready = true;
     return RT_OK;
 }
@@ -619,8 +640,81 @@ struct Segment {       // a contiguous piece of one tensor inside one chunk
 };
 }  // namespace
 
-int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
-                     uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems, void* stream_) {
+// Cuts the tensor list into chunks of at most chunk_elems staged elements.  A tensor may span
+// chunks; every piece starts at a multiple of 8 elements, both inside its tensor (so the Philox
+// blocks line up) and inside the staging buffers (so 128-bit accesses stay aligned).
+static void cut_into_chunks(const rt_tensor_desc* descs, uint32_t n, uint64_t chunk_elems,
+                            std::vector<std::vector<Segment>>& chunks) {
+    std::vector<Segment> cur;
+    uint64_t used = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        uint64_t done = 0;
+        const uint64_t numel = descs[i].numel;
+        while (done < numel) {
+            if (used >= chunk_elems) {
+                chunks.push_back(std::move(cur));
+                cur.clear();
+                used = 0;
+            }
+            const uint64_t take = std::min(numel - done, chunk_elems - used);
+            cur.push_back(Segment{i, done, take, used});
+            done += take;
+            used = align_up(used + take, kVec);  // next piece starts 16-byte aligned
+        }
+    }
+    if (!cur.empty()) chunks.push_back(std::move(cur));
+}
+
+int rt_streamed_plan(const rt_tensor_desc* descs, uint32_t n, uint64_t chunk_elems, uint64_t* out, uint32_t cap,
+                     uint32_t* n_out) {
+    if (!n_out) return fail(RT_EINVAL, "n_out is NULL");
+    if (n > 0 && !descs) return fail(RT_EINVAL, "descs is NULL");
+    if (chunk_elems < kVec || (chunk_elems % kVec) != 0)
+        return fail(RT_EINVAL, "chunk_elems %llu must be a positive multiple of 8", (unsigned long long)chunk_elems);
+    std::vector<std::vector<Segment>> chunks;
+    cut_into_chunks(descs, n, chunk_elems, chunks);
+    uint32_t k = 0;
+    for (size_t c = 0; c < chunks.size(); ++c)
+        for (const Segment& s : chunks[c]) {
+            if (out && k < cap) {
+                uint64_t* row = out + 5 * (size_t)k;
+                row[0] = c; row[1] = s.tensor; row[2] = s.start; row[3] = s.count; row[4] = s.stage_off;
+            }
+            ++k;
+        }
+    *n_out = k;
+    return RT_OK;
+}
+
+// Retires finished tickets (non-blocking).
+static int streamed_poll(Streamed& st) {
+    while (!st.ticket_events.empty()) {
+        hipError_t e = hipEventQuery(st.ticket_events.front().second);
+        if (e == hipErrorNotReady) break;
+        if (e != hipSuccess) return fail(RT_EHIP, "hipEventQuery failed: %s", hipGetErrorString(e));
+        st.tickets_done = st.ticket_events.front().first;
+        st.event_pool.push_back(st.ticket_events.front().second);
+        st.ticket_events.pop_front();
+    }
+    return RT_OK;
+}
+
+static int streamed_wait(rt_handle* h) {
+    Streamed& st = h->st;
+    if (!st.ready) return RT_OK;
+    HIP_TRY(hipSetDevice(h->device));
+    HIP_TRY(hipStreamSynchronize(st.d2h));
+    HIP_TRY(hipStreamSynchronize(st.comp));
+    HIP_TRY(hipStreamSynchronize(st.h2d));
+    st.pending = false;
+    for (auto& r : st.ring) r.in_flight = false;
+    return streamed_poll(st);
+}
+
+// Validates and enqueues the whole pipeline of one call; does not wait for it.
+static int streamed_enqueue(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
+                            uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems, void* stream_,
+                            bool trace, uint64_t* ticket_out) {
     if (!h) return fail(RT_EINVAL, "handle is NULL");
     int rc = validate(descs, n, scalars, n_scalars, noise_mode, /*allow_host=*/true);
     if (rc != RT_OK) return rc;
@@ -632,36 +726,17 @@ int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, cons
     for (uint32_t i = 0; i < n; ++i)
         if (descs[i].row_mean && scalars[descs[i].scalars_idx].centralization != 0.0f && descs[i].row_len == 0)
             return fail(RT_EINVAL, "tensor %u: row_len is 0", i);
-    if (n == 0) return RT_OK;
     hipStream_t user = (hipStream_t)stream_;
     HIP_TRY(hipSetDevice(h->device));
     rc = streamed_init(h);
     if (rc != RT_OK) return rc;
     Streamed& st = h->st;
-    const auto wall0 = std::chrono::steady_clock::now();
+    if (ticket_out) *ticket_out = st.tickets_issued;  // nothing to wait for beyond what is already issued
+    if (n == 0) return RT_OK;
 
     // ---- cut the tensor list into chunks of at most chunk_elems staged elements
     std::vector<std::vector<Segment>> chunks;
-    {
-        std::vector<Segment> cur;
-        uint64_t used = 0;
-        for (uint32_t i = 0; i < n; ++i) {
-            uint64_t done = 0;
-            const uint64_t numel = descs[i].numel;
-            while (done < numel) {
-                if (used >= chunk_elems) {
-                    chunks.push_back(std::move(cur));
-                    cur.clear();
-                    used = 0;
-                }
-                const uint64_t take = std::min(numel - done, chunk_elems - used);
-                cur.push_back(Segment{i, done, take, used});
-                done += take;
-                used = align_up(used + take, kVec);  // next piece starts 16-byte aligned
-            }
-        }
-        if (!cur.empty()) chunks.push_back(std::move(cur));
-    }
+    cut_into_chunks(descs, n, chunk_elems, chunks);
 
     // ---- staging buffers sized for the widest element type that is host resident
     int stage_esize[4] = {0, 0, 0, 0};
@@ -679,7 +754,12 @@ int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, cons
     for (int a = 0; a < 4; ++a)
         for (int b = 0; b < 2; ++b)
             if (stage_esize[a]) {
-                rc = dev_reserve(st.stage[a][b], max_used * 4);  // sized for fp32 so dtype changes never realloc
+                const size_t want = max_used * 4;  // sized for fp32 so dtype changes never realloc
+                if (want > st.stage[a][b].cap && st.pending) {
+                    rc = streamed_wait(h);  // the buffer may be in use by an earlier asynchronous call
+                    if (rc != RT_OK) return rc;
+                }
+                rc = dev_reserve(st.stage[a][b], want);
                 if (rc != RT_OK) return rc;
             }
 
@@ -690,7 +770,7 @@ int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, cons
     std::vector<size_t> plan_off(chunks.size());
     std::vector<uint8_t> blob;
     for (size_t c = 0; c < chunks.size(); ++c) {
-        const int b = (int)(c & 1);
+        const int b = (int)((st.seq + c) & 1);
         for (const Segment& s : chunks[c]) {
             const rt_tensor_desc& d = descs[s.tensor];
             rt_tensor_desc q = d;
@@ -719,29 +799,34 @@ int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, cons
         blob.resize(plan_off[c] + plans[c].bytes);
         if (plans[c].bytes) memcpy(blob.data() + plan_off[c], h->image.data(), plans[c].bytes);
     }
-    if (blob.size() > st.tables_host_cap) {
-        if (st.tables_host) HIP_TRY(hipHostFree(st.tables_host));
-        st.tables_host = nullptr;
-        st.tables_host_cap = 0;
-        const size_t want = blob.size() + blob.size() / 4 + 4096;
-        hipError_t e = hipHostMalloc(&st.tables_host, want, hipHostMallocDefault);
-        if (e != hipSuccess) return fail(RT_ENOMEM, "hipHostMalloc(%zu) failed: %s", want, hipGetErrorString(e));
-        st.tables_host_cap = want;
+    Streamed::TableRing& tab = st.ring[st.ring_pos++ % 4];
+    if (tab.in_flight) {
+        HIP_TRY(hipEventSynchronize(tab.done));
+        tab.in_flight = false;
     }
-    rc = dev_reserve(st.tables, blob.size());
+    if (blob.size() > tab.host_cap) {
+        if (tab.host) HIP_TRY(hipHostFree(tab.host));
+        tab.host = nullptr;
+        tab.host_cap = 0;
+        const size_t want = blob.size() + blob.size() / 4 + 4096;
+        hipError_t e = hipHostMalloc(&tab.host, want, hipHostMallocDefault);
+        if (e != hipSuccess) return fail(RT_ENOMEM, "hipHostMalloc(%zu) failed: %s", want, hipGetErrorString(e));
+        tab.host_cap = want;
+    }
+    rc = dev_reserve(tab.dev, blob.size());
     if (rc != RT_OK) return rc;
-    memcpy(st.tables_host, blob.data(), blob.size());
+    memcpy(tab.host, blob.data(), blob.size());
 
     // grads (and anything else already queued by the caller) must be ready
     HIP_TRY(hipEventRecord(st.start, user));
     HIP_TRY(hipStreamWaitEvent(st.h2d, st.start, 0));
     HIP_TRY(hipStreamWaitEvent(st.comp, st.start, 0));
     if (!blob.empty())
-        HIP_TRY(hipMemcpyAsync(st.tables.ptr, st.tables_host, blob.size(), hipMemcpyHostToDevice, st.comp));
+        HIP_TRY(hipMemcpyAsync(tab.dev.ptr, tab.host, blob.size(), hipMemcpyHostToDevice, st.comp));
 
     st.bytes_h2d = st.bytes_d2h = 0;
     st.timeline.clear();
-    const bool trace = h->timing;
+    st.pending = true;
     if (trace) {
         while (st.tl_events.size() < 4 * chunks.size()) {
             hipEvent_t e;
@@ -749,12 +834,11 @@ int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, cons
             st.tl_events.push_back(e);
         }
     }
-    bool used_buf[2] = {false, false};
     for (size_t c = 0; c < chunks.size(); ++c) {
-        const int b = (int)(c & 1);
+        const int b = (int)((st.seq + c) & 1);
         const auto& segs = chunks[c];
         // H2D: the buffer is free once the D2H of the chunk two back has finished
-        if (used_buf[b]) HIP_TRY(hipStreamWaitEvent(st.h2d, st.d2h_done[b], 0));
+        if (st.used_buf[b]) HIP_TRY(hipStreamWaitEvent(st.h2d, st.d2h_done[b], 0));
         if (trace) HIP_TRY(hipEventRecord(st.tl_events[4 * c + 0], st.h2d));
         for (size_t k = 0; k < segs.size(); ++k) {
             const Segment& s = segs[k];
@@ -776,7 +860,7 @@ int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, cons
 
         // compute
         HIP_TRY(hipStreamWaitEvent(st.comp, st.h2d_done[b], 0));
-        rc = enqueue_kernels(plans[c], (const uint8_t*)st.tables.ptr + plan_off[c], seed, noise_mode, nullptr,
+        rc = enqueue_kernels(plans[c], (const uint8_t*)tab.dev.ptr + plan_off[c], seed, noise_mode, nullptr,
                              nullptr, st.comp);
         if (rc != RT_OK) return rc;
         HIP_TRY(hipEventRecord(st.comp_done[b], st.comp));
@@ -800,19 +884,64 @@ int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, cons
         }
         if (trace) HIP_TRY(hipEventRecord(st.tl_events[4 * c + 3], st.d2h));
         HIP_TRY(hipEventRecord(st.d2h_done[b], st.d2h));
-        used_buf[b] = true;
+        st.used_buf[b] = true;
     }
-    // Host memory is final on return; device-resident arrays are final for the caller's stream.
-    HIP_TRY(hipStreamSynchronize(st.d2h));
-    HIP_TRY(hipStreamSynchronize(st.comp));
-    st.seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - wall0).count();
-    if (trace) {
-        st.timeline.resize(4 * chunks.size());
-        for (size_t i = 0; i < st.timeline.size(); ++i)
-            HIP_TRY(hipEventElapsedTime(&st.timeline[i], st.tl_events[0], st.tl_events[i]));
+    st.seq += chunks.size();
+    HIP_TRY(hipEventRecord(tab.done, st.comp));
+    tab.in_flight = true;
+    // ticket: completes when the last D2H of this call has landed (D2H follows compute, so
+    // device-resident arrays are final by then as well)
+    hipEvent_t te;
+    if (!st.event_pool.empty()) {
+        te = st.event_pool.back();
+        st.event_pool.pop_back();
+    } else {
+        HIP_TRY(hipEventCreateWithFlags(&te, hipEventDisableTiming));
     }
+    HIP_TRY(hipEventRecord(te, st.d2h));
+    st.ticket_events.emplace_back(++st.tickets_issued, te);
+    if (ticket_out) *ticket_out = st.tickets_issued;
+    if (trace) st.timeline.assign(4 * chunks.size(), 0.0f);
     return RT_OK;
 }
+
+int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
+                     uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems, void* stream) {
+    if (!h) return fail(RT_EINVAL, "handle is NULL");
+    const auto wall0 = std::chrono::steady_clock::now();
+    const bool trace = h->timing;
+    int rc = streamed_enqueue(h, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, stream, trace, nullptr);
+    if (rc != RT_OK) return rc;
+    // Host memory is final on return; device-resident arrays are final for the caller's stream.
+    rc = streamed_wait(h);
+    if (rc != RT_OK) return rc;
+    Streamed& st = h->st;
+    st.seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - wall0).count();
+    if (trace)
+        for (size_t i = 0; i < st.timeline.size(); ++i)
+            HIP_TRY(hipEventElapsedTime(&st.timeline[i], st.tl_events[0], st.tl_events[i]));
+    return RT_OK;
+}
+
+int rt_step_streamed_async(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
+                           uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems, void* stream,
+                           uint64_t* ticket) {
+    if (!h) return fail(RT_EINVAL, "handle is NULL");
+    return streamed_enqueue(h, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, stream, false, ticket);
+}
+
+int rt_streamed_wait(rt_handle* h) {
+    if (!h) return fail(RT_EINVAL, "handle is NULL");
+    return streamed_wait(h);
+}
+
+int rt_streamed_completed(rt_handle* h, uint64_t* ticket_done) {
+    if (!h || !ticket_done) return fail(RT_EINVAL, "NULL argument");
+    int rc = streamed_poll(h->st);
+    *ticket_done = h->st.tickets_done;
+    return rc;
+}
+
 
 int rt_streamed_timeline(rt_handle* h, float* out, uint32_t cap, uint32_t* n_out) {
     if (!h || !n_out) return fail(RT_EINVAL, "NULL argument");

@@ -174,16 +174,24 @@ def step_resident(handle: N.Handle, entries: Sequence[Entry], scalars: Sequence[
 
 
 def step_streamed(handle: N.Handle, entries: Sequence[Entry], scalars: Sequence[N.RtScalars], *, seed: int,
-                  explicit_noise: bool, chunk_elems: int, stream: Optional[int] = None) -> None:
-    """Chunked H2D / update / D2H for tensors with CPU-resident arrays.  Host
-    memory is final when this returns."""
+                  explicit_noise: bool, chunk_elems: int, stream: Optional[int] = None,
+                  wait: bool = True) -> Optional[int]:
+    """Chunked H2D / update / D2H for tensors with CPU-resident arrays.  With
+    ``wait`` (default) host memory is final when this returns.  Without it the
+    call only enqueues and returns a ticket: until ``handle.streamed_completed()``
+    reaches it (or ``handle.streamed_wait()`` returns) the caller must keep the
+    tensors alive and leave p / m / v alone."""
     if not entries:
-        return
+        return None
     d = pack_descs(entries, streamed=True)
     if stream is None:
         stream = torch.cuda.current_stream(handle.device).cuda_stream
-    handle.step_streamed(_descs_ptr(d), len(entries), scalars_array(scalars), len(scalars), seed & (2 ** 64 - 1),
-                         N.RT_NOISE_EXPLICIT if explicit_noise else N.RT_NOISE_PHILOX, int(chunk_elems), stream)
+    args = (_descs_ptr(d), len(entries), scalars_array(scalars), len(scalars), seed & (2 ** 64 - 1),
+            N.RT_NOISE_EXPLICIT if explicit_noise else N.RT_NOISE_PHILOX, int(chunk_elems), stream)
+    if wait:
+        handle.step_streamed(*args)
+        return None
+    return handle.step_streamed_async(*args)
 
 
 def grad_norm(handle: N.Handle, grads: Sequence[torch.Tensor], *, inv_loss_scale: float = 1.0,

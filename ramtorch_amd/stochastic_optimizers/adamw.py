@@ -110,6 +110,10 @@ class AdamW(Optimizer):
         self.loss_scale = float(loss_scale)
         self.max_grad_norm = max_grad_norm
         self.last_grad_norm: Optional[torch.Tensor] = None  # [norm, clip_coef, found_inf bits, -] on the GPU
+        self.fuse_in_backward = True      # the hook of make_post_accumulate_hook() is live
+        self.max_inflight_bytes = 2 << 30  # gradients kept alive for updates still in flight (step_param)
+        self._stepped_early = set()       # id(param) updated by step_param since the last step()
+        self._inflight = []               # (device, ticket, bytes, tensors kept alive)
         # eager state allocation, as adamw.py:84-104
         for group in self.param_groups:
             for p in group["params"]:
@@ -119,6 +123,42 @@ class AdamW(Optimizer):
     def __setstate__(self, state):
         # load_state_dict (and unpickling) replace self.state wholesale: drop everything derived from it
         super().__setstate__(state)
+        self._recs = None
+        self._desc_cache = {}
+
+    def state_dict(self):
+        """Same layout as the reference (``state`` with ``step / ema / ema_squared`` per
+        parameter index, ``param_groups``) plus one extra top-level entry with the Philox
+        seed, so that a resumed run draws the noise it would have drawn.  torch's loader
+        ignores entries it does not know, so the reference can read these checkpoints."""
+        sd = super().state_dict()
+        sd["ramtorch_amd"] = {"seed": self.seed}
+        return sd
+
+    def load_state_dict(self, state_dict):
+        """torch's loader casts ``ema`` / ``ema_squared`` to the parameter's dtype and
+        device and drops pinning, which would silently undo ``dtype=`` /
+        ``storage_device=``.  After it has restored steps and hyper-parameters, the two
+        states are taken again from the checkpoint itself: original dtype, placed on
+        ``storage_device`` (pinned when that is the CPU)."""
+        super().load_state_dict(state_dict)
+        extra = state_dict.get("ramtorch_amd")
+        if isinstance(extra, dict) and "seed" in extra:
+            self.seed = int(extra["seed"])
+        saved_ids = [i for g in state_dict["param_groups"] for i in g["params"]]
+        ours = [p for g in self.param_groups for p in g["params"]]
+        for idx, p in zip(saved_ids, ours):
+            saved = state_dict["state"].get(idx)
+            if saved is None:
+                continue
+            st = self.state[p]
+            for k in ("ema", "ema_squared"):
+                if k in saved and torch.is_tensor(saved[k]):
+                    t = saved[k].detach().to(device=self.optim_state_device).clone(
+                        memory_format=torch.contiguous_format)
+                    if self.optim_state_device == "cpu" and torch.cuda.is_available():
+                        t = t.pin_memory()
+                    st[k] = t
         self._recs = None
         self._desc_cache = {}
 
@@ -176,10 +216,12 @@ class AdamW(Optimizer):
             return recs
         k = 0
         recs = []
-        for g in groups:
+        self._positions = {}
+        for gi, g in enumerate(groups):
             row = []
-            for p in g["params"]:
+            for j, p in enumerate(g["params"]):
                 row.append(self._make_rec(p, k))
+                self._positions[id(p)] = (gi, j)
                 k += 1
             recs.append(row)
         self._recs = recs
@@ -208,6 +250,8 @@ class AdamW(Optimizer):
             raise RuntimeError("ramtorch_amd.AdamW.step needs a GPU: the update runs only as HIP kernels")
 
         recs = self._records()
+        self.finish_early_steps()  # updates started from the backward hook must have landed
+        early = self._stepped_early
         scalars: List[N.RtScalars] = []
         scalar_key: Dict[tuple, int] = {}
         # plain lane: tensors wholly on one GPU, contiguous, nothing special -> columns only
@@ -230,6 +274,8 @@ class AdamW(Optimizer):
                     grad = grads.get(p, p.grad) if grads is not None else p.grad
                     if grad is None:
                         continue  # adamw.py:114: skipped, and its step count does not advance
+                    if early and id(p) in early:
+                        continue  # already updated by step_param() during this backward
                     if grad.is_sparse:
                         raise RuntimeError("AdamW does not support sparse gradients")  # adamw.py:118-119
                     r = row[k]
@@ -329,7 +375,101 @@ class AdamW(Optimizer):
                                         chunk_elems=chunk_elems)
             for dst, tmp in writeback:
                 dst.copy_(tmp)
+        early.clear()
         return loss
+
+    # -- updating one parameter as soon as its gradient exists --------------------------------
+    def make_post_accumulate_hook(self):
+        """A callable for ramtorch's ``_ramtorch_post_accumulate_grad_hooks``
+        (``linear.py:97-111``: called as ``hook(param)`` inside ``Linear.backward`` while
+        ``param.ramtorch_grad`` holds the accumulated gradient on the GPU).  It runs the
+        update of that parameter right there, from the GPU gradient, instead of waiting
+        for ``step()`` to ship the gradient back from the CPU (``adamw.py:167``).  Set
+        ``optimizer.fuse_in_backward = False`` during gradient-accumulation micro-steps.
+        ``step()`` afterwards waits for these updates and skips the parameters they covered."""
+        def hook(param):
+            if self.fuse_in_backward:
+                grad = getattr(param, "ramtorch_grad", None)
+                self.step_param(param, grad if grad is not None else param.grad)
+        return hook
+
+    def step_param(self, p: torch.Tensor, grad: Optional[torch.Tensor] = None) -> None:
+        """Update one parameter now, without waiting: same arithmetic, same noise and same
+        ``state["step"]`` bookkeeping as ``step()`` would apply to it.  The update is queued
+        behind the work already on the current stream; host-resident arrays are final after
+        ``finish_early_steps()`` (``step()`` calls it)."""
+        N.lib()
+        if not torch.cuda.is_available():
+            raise RuntimeError("ramtorch_amd.AdamW.step_param needs a GPU: the update runs only as HIP kernels")
+        if grad is None:
+            grad = p.grad
+        if grad is None:
+            return
+        if grad.is_sparse:
+            raise RuntimeError("AdamW does not support sparse gradients")
+        if self.max_grad_norm is not None:
+            raise NotImplementedError("step_param with max_grad_norm (the global norm needs every gradient)")
+        if id(p) in self._stepped_early:
+            raise RuntimeError("step_param called twice for one parameter without a step() in between")
+        recs = self._records()
+        pos = self._positions.get(id(p))
+        if pos is None:
+            raise ValueError("step_param: tensor is not a parameter of this optimizer")
+        gi, k = pos
+        group = self.param_groups[gi]
+        if group["centralization"] != 0:
+            raise NotImplementedError("step_param with centralization")
+        r = recs[gi][k]
+        state = r.state
+        if (state.get("ema") is not r.m or state.get("ema_squared") is not r.v or p.data_ptr() != r.p_ptr
+                or r.m.data_ptr() != r.m_ptr or r.v.data_ptr() != r.v_ptr):
+            r = recs[gi][k] = self._make_rec(p, r.tensor_id)
+            state = r.state
+        if not (p.is_contiguous() and r.m.is_contiguous() and r.v.is_contiguous()):
+            raise NotImplementedError("step_param needs contiguous parameter and state tensors")
+        dev = r.dev
+        with torch.no_grad():
+            g = grad.detach()
+            if not g.is_cuda or g.device.index != dev:
+                g = g.to(f"cuda:{dev}", non_blocking=True)
+            if not g.is_contiguous():
+                g = g.contiguous()
+            if g.dtype not in (torch.bfloat16, torch.float32, torch.float16):
+                g = g.to(torch.float32)
+            step = state["step"] + 1
+            state["step"] = step
+            inv_loss_scale = 1.0 / self.loss_scale if self.loss_scale != 1.0 else 1.0
+            sc = [F.make_scalars(group["lr"], tuple(group["betas"]), group["eps"], group["weight_decay"], step,
+                                 inv_loss_scale=inv_loss_scale)]
+            e = F.Entry(p=p.data, g=g, m=r.m, v=r.v, step=step, scalars_idx=0, tensor_id=r.tensor_id)
+            h = _handle(dev)
+            with torch.cuda.device(dev):
+                if e.p.is_cuda and e.m.is_cuda and e.v.is_cuda:
+                    F.step_resident(h, [e], sc, seed=self.seed, explicit_noise=False)  # stream-ordered already
+                else:
+                    chunk_elems = max(8, (self.stream_chunk_bytes // 2) // 8 * 8)
+                    ticket = F.step_streamed(h, [e], sc, seed=self.seed, explicit_noise=False,
+                                             chunk_elems=chunk_elems, wait=False)
+                    self._inflight.append((dev, ticket, g.numel() * g.element_size(), (g, e)))
+                    self._release_finished(dev)
+        self._stepped_early.add(id(p))
+
+    def _release_finished(self, dev: int) -> None:
+        """Drop the references of finished asynchronous updates; if too many gradient bytes
+        are still held, wait for the pipeline."""
+        h = _handle(dev)
+        done = h.streamed_completed()
+        self._inflight = [x for x in self._inflight if not (x[0] == dev and x[1] <= done)]
+        if sum(x[2] for x in self._inflight) > self.max_inflight_bytes:
+            h.streamed_wait()
+            self._inflight = [x for x in self._inflight if x[0] != dev]
+
+    def finish_early_steps(self) -> None:
+        """Wait until every update started by ``step_param`` has landed in host memory."""
+        for dev in sorted({x[0] for x in self._inflight}):
+            with torch.cuda.device(dev):
+                _handle(dev).streamed_wait()
+        self._inflight = []
 
     def _plain_descs(self, dev: int, lane) -> np.ndarray:
         """Descriptor array of the plain lane.  The columns that describe p / m / v are

@@ -148,3 +148,123 @@ def test_optimizer_gpu_params_with_default_cpu_states():
     torch.cuda.synchronize()
     np.testing.assert_array_equal(bits16(P), po)
     np.testing.assert_array_equal(bits16(opt.state[P]["ema"]), mo)
+
+
+# ---- updates started from inside backward (the post-accumulate-grad hook of ramtorch.Linear) ----------
+def _offload_params(shapes, seed):
+    ps, gs, refs = [], [], []
+    for i, shp in enumerate(shapes):
+        n = int(np.prod(shp))
+        p, g, _, _ = oracle.synth_inputs(n, seed + i)
+        t = torch.nn.Parameter(host16(p).view(shp))
+        t.is_ramtorch = True
+        ps.append(t)
+        gs.append(g)
+        refs.append([p.copy(), np.zeros(n, np.uint16), np.zeros(n, np.uint16)])
+    return ps, gs, refs
+
+
+def test_post_accumulate_hook_updates_from_the_gpu_gradient():
+    shapes = [(256, 128), (128,), (64, 64), (40_000,)]
+    ps, gs, refs = _offload_params(shapes, 1200)
+    opt = ramtorch_amd.AdamW(ps, seed=31, stream_chunk_bytes=32_768, **HP0)
+    hook = opt.make_post_accumulate_hook()
+    for step in (1, 2):
+        # what Linear.backward does per layer, last layer first (linear.py:341-430)
+        for p, g in reversed(list(zip(ps, gs))):
+            p.ramtorch_grad = dev16(g).view(p.shape)          # accumulated gradient, on the GPU
+            hook(p)
+            cpu_grad = p.ramtorch_grad.to("cpu", non_blocking=True)
+            del p.ramtorch_grad
+            p.grad = cpu_grad                                  # the reference still ships it to the CPU
+        assert all(opt.state[p]["step"] == step for p in ps)
+        opt.step()                                             # waits; must not apply the update twice
+        sco = oracle.scalars_from_hparams(step=step, **HP0)
+        for i, (p, g) in enumerate(zip(ps, gs)):
+            oracle.step_tensor(refs[i][0], g, refs[i][1], refs[i][2], sco, seed=31, step=step, tensor_id=i)
+            np.testing.assert_array_equal(bits16(p), refs[i][0], err_msg=f"step {step} param {i}")
+            np.testing.assert_array_equal(bits16(opt.state[p]["ema"]), refs[i][1])
+            np.testing.assert_array_equal(bits16(opt.state[p]["ema_squared"]), refs[i][2])
+            assert opt.state[p]["step"] == step
+    # with the hook switched off (gradient-accumulation micro-step) nothing happens until step()
+    opt.fuse_in_backward = False
+    for p, g in zip(ps, gs):
+        p.ramtorch_grad = dev16(g).view(p.shape)
+        hook(p)
+        del p.ramtorch_grad
+        p.grad = host16(g, pin=False).view(p.shape)
+    assert all(opt.state[p]["step"] == 2 for p in ps)
+    opt.step()
+    sco = oracle.scalars_from_hparams(step=3, **HP0)
+    for i, (p, g) in enumerate(zip(ps, gs)):
+        oracle.step_tensor(refs[i][0], g, refs[i][1], refs[i][2], sco, seed=31, step=3, tensor_id=i)
+        np.testing.assert_array_equal(bits16(p), refs[i][0], err_msg=f"step 3 param {i}")
+
+
+def test_step_param_mixes_with_step_and_rejects_double_use():
+    ps, gs, refs = _offload_params([(3000,), (5000,)], 1300)
+    gpu_p, gpu_g, _, _ = oracle.synth_inputs(7000, 1310)
+    q = torch.nn.Parameter(dev16(gpu_p))                       # a GPU-resident parameter in the same optimizer
+    opt = ramtorch_amd.AdamW([{"params": ps}, {"params": [q], "lr": 3e-4}], seed=2, storage_device="cpu", **HP0)
+    opt.state[q]["ema"] = opt.state[q]["ema"].cuda()
+    opt.state[q]["ema_squared"] = opt.state[q]["ema_squared"].cuda()
+    opt.step_param(ps[0], dev16(gs[0]))                        # early
+    opt.step_param(q, dev16(gpu_g))                            # early, resident
+    with pytest.raises(RuntimeError, match="twice"):
+        opt.step_param(ps[0], dev16(gs[0]))
+    ps[1].grad = host16(gs[1], pin=False)                      # this one waits for step()
+    ps[0].grad = host16(gs[0], pin=False)
+    opt.step()
+    torch.cuda.synchronize()
+    sco = oracle.scalars_from_hparams(step=1, **HP0)
+    for i in (0, 1):
+        oracle.step_tensor(refs[i][0], gs[i], refs[i][1], refs[i][2], sco, seed=2, step=1, tensor_id=i)
+        np.testing.assert_array_equal(bits16(ps[i]), refs[i][0], err_msg=f"param {i}")
+    qo, mo, vo = gpu_p.copy(), np.zeros(7000, np.uint16), np.zeros(7000, np.uint16)
+    hp = dict(HP0, lr=3e-4)
+    oracle.step_tensor(qo, gpu_g, mo, vo, oracle.scalars_from_hparams(step=1, **hp), seed=2, step=1, tensor_id=2)
+    np.testing.assert_array_equal(bits16(q), qo)
+    with pytest.raises(ValueError):
+        opt.step_param(torch.nn.Parameter(torch.zeros(4)), torch.zeros(4))
+
+
+def test_async_calls_chain_through_the_shared_staging_buffers(handle):
+    """Many asynchronous single-tensor calls in a row, sizes that do not divide the
+    chunk: buffers alternate across calls and a grown staging buffer is handled."""
+    sc, sco = F.make_scalars(step=5, **HP0), oracle.scalars_from_hparams(step=5, **HP0)
+    lens = [100, 9000, 70_001, 8192, 33, 250_000, 4096, 12_345]
+    entries, inputs, tickets = [], [], []
+    for i, n in enumerate(lens):
+        p, g, m, v = oracle.synth_inputs(n, 1400 + i)
+        e = F.Entry(p=host16(p), g=dev16(g), m=host16(m), v=host16(v), step=5, scalars_idx=0, tensor_id=i)
+        entries.append(e)
+        inputs.append((p, g, m, v))
+        tickets.append(F.step_streamed(handle, [e], [sc], seed=8, explicit_noise=False, chunk_elems=16_384,
+                                       wait=False))
+    assert tickets == sorted(tickets) and len(set(tickets)) == len(tickets)
+    handle.streamed_wait()
+    assert handle.streamed_completed() == tickets[-1]
+    for i, (e, (p, g, m, v)) in enumerate(zip(entries, inputs)):
+        po, mo, vo = p.copy(), m.copy(), v.copy()
+        oracle.step_tensor(po, g, mo, vo, sco, seed=8, step=5, tensor_id=i)
+        for name, t, a in zip("pmv", (e.p, e.m, e.v), (po, mo, vo)):
+            np.testing.assert_array_equal(bits16(t), a, err_msg=f"tensor {i} (n={lens[i]}) {name}")
+
+
+def test_load_state_dict_restores_pinned_host_states():
+    import copy
+    ps, gs, _ = _offload_params([(64, 32)], 1500)
+    a = ramtorch_amd.AdamW(ps, seed=3, **HP0)
+    ps[0].grad = host16(gs[0], pin=False).view(64, 32)
+    a.step()
+    sd = copy.deepcopy(a.state_dict())
+    ps2 = [torch.nn.Parameter(ps[0].detach().clone().pin_memory())]
+    b = ramtorch_amd.AdamW(ps2, **HP0)
+    b.load_state_dict(sd)
+    st = b.state[ps2[0]]
+    assert st["ema"].is_pinned() and st["ema_squared"].is_pinned() and b.seed == 3 and st["step"] == 1
+    for opt, params in ((a, ps), (b, ps2)):
+        params[0].grad = host16(gs[0], pin=False).view(64, 32)
+        opt.step()
+    assert nmis(ps[0].detach(), ps2[0].detach()) == 0
+    assert nmis(a.state[ps[0]]["ema_squared"], st["ema_squared"]) == 0

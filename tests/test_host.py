@@ -145,13 +145,35 @@ def test_state_dict_round_trip_keeps_reference_keys():
     opt.state[ps[0]]["step"] = 7
     opt.state[ps[0]]["ema"].fill_(0.5)
     sd = opt.state_dict()
-    assert set(sd) == {"state", "param_groups"}
+    assert set(sd) == {"state", "param_groups", "ramtorch_amd"}
     assert set(sd["state"][0]) == {"step", "ema", "ema_squared"}
     opt2 = ramtorch_amd.AdamW(_params(), lr=1e-3)
     opt2.load_state_dict(sd)
     p0 = opt2.param_groups[0]["params"][0]
     assert opt2.state[p0]["step"] == 7 and opt2.param_groups[0]["lr"] == 2e-3
     assert torch.equal(opt2.state[p0]["ema"], torch.full((4, 6), 0.5, dtype=torch.bfloat16))
+
+
+def test_load_state_dict_keeps_state_dtype_device_and_seed():
+    ps = [torch.nn.Parameter(torch.zeros(8, dtype=torch.bfloat16))]
+    a = ramtorch_amd.AdamW(ps, dtype=torch.float32, seed=77)
+    a.state[ps[0]]["ema_squared"].fill_(1.0 + 2.0 ** -20)      # not representable in bf16
+    a.state[ps[0]]["step"] = 3
+    sd = a.state_dict()
+    assert sd["ramtorch_amd"] == {"seed": 77} and set(sd["state"][0]) == {"step", "ema", "ema_squared"}
+    b = ramtorch_amd.AdamW([torch.nn.Parameter(torch.zeros(8, dtype=torch.bfloat16))], dtype=torch.float32)
+    b.load_state_dict(sd)
+    st = b.state[b.param_groups[0]["params"][0]]
+    assert st["ema_squared"].dtype == torch.float32 and st["ema_squared"].device.type == "cpu"
+    assert float(st["ema_squared"][0]) == 1.0 + 2.0 ** -20 and st["step"] == 3 and b.seed == 77
+    assert st["ema_squared"].data_ptr() != a.state[ps[0]]["ema_squared"].data_ptr()   # a copy, not an alias
+    # a checkpoint written by the reference (no extra entry) loads and keeps the current seed
+    del sd["ramtorch_amd"]
+    c = ramtorch_amd.AdamW([torch.nn.Parameter(torch.zeros(8, dtype=torch.bfloat16))], seed=5)
+    c.load_state_dict(sd)
+    assert c.seed == 5
+    # and torch's own loader accepts ours
+    torch.optim.SGD([torch.nn.Parameter(torch.zeros(8))], lr=0.1).state_dict()
 
 
 def test_step_without_gpu_raises_and_leaves_state_alone():
@@ -206,3 +228,37 @@ def test_build_module_knows_its_sources():
     assert "--offload-arch=gfx950" in build.HIPCC_FLAGS and "-ffp-contract=off" in build.HIPCC_FLAGS
     i = build.HIPCC_FLAGS.index("-packed-fp32-ops")
     assert build.HIPCC_FLAGS[i - 3:i] == ["-Xclang", "-target-feature", "-Xclang"]
+
+
+# ---- chunk schedule of the streamed path (pure host logic) -----------------------------------
+@pytest.mark.parametrize("chunk_elems", [8, 64, 8192, 100_000, 1 << 27])
+def test_streamed_chunk_schedule_covers_every_element_once(chunk_elems):
+    rng = np.random.default_rng(chunk_elems)
+    lens = [0, 1, 7, 8, 9, 4096, 8191, 8193, 250_007, 16, 0, 5] + [int(x) for x in rng.integers(1, 50_000, 20)]
+    d = np.zeros(len(lens), F.DESC_DTYPE)
+    d["numel"] = lens
+    plan = N.streamed_plan(d.ctypes.data_as(ctypes.POINTER(N.RtTensorDesc)), len(lens), chunk_elems)
+    covered = [0] * len(lens)
+    per_chunk = {}
+    last = (-1, -1)
+    for chunk, tensor, start, count, off in plan:
+        assert count > 0 and start % 8 == 0 and off % 8 == 0          # Philox blocks and 16-byte alignment
+        assert start == covered[tensor], "pieces of a tensor must be consecutive"
+        assert (chunk, tensor) >= last                                  # tensors in order, chunks in order
+        last = (chunk, tensor)
+        covered[tensor] += count
+        lo, hi = per_chunk.get(chunk, (0, 0))
+        assert off >= hi, "pieces overlap inside the staging buffer"
+        per_chunk[chunk] = (lo, off + count)
+        assert off + count <= chunk_elems
+    assert covered == lens
+    assert sorted(per_chunk) == list(range(len(per_chunk)))
+    # no chunk but the last may be left mostly empty: a new chunk starts only when the previous one is full
+    for c in sorted(per_chunk)[:-1]:
+        assert per_chunk[c][1] > chunk_elems - 8
+
+
+def test_streamed_plan_rejects_bad_chunk_size():
+    d = np.zeros(1, F.DESC_DTYPE)
+    with pytest.raises(N.NativeError):
+        N.streamed_plan(d.ctypes.data_as(ctypes.POINTER(N.RtTensorDesc)), 1, 12)
