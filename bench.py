@@ -27,6 +27,10 @@ ema~N(0,1e-4), ema_squared=N(0,1e-3)^2, stored bf16):
             by 1024 and unscaled in-kernel, global-norm clip to 1.0
   streamed  Llama-3-8B shapes with p/ema/ema_squared in pinned host memory,
             bf16 grads on the GPU, 256 MB chunks (--stream-gb bounds the host set)
+  hooked    the same set, but each tensor is updated by AdamW.step_param() as a
+            backward pass would hand its gradient over (last tensor first), and
+            step() only waits: the grad hand-off from ramtorch.Linear's
+            post-accumulate hook
 """
 from __future__ import annotations
 
@@ -170,7 +174,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="llama8b", choices=["llama8b", "cfg0", "small", "mixed", "streamed"])
+    ap.add_argument("--workload", default="llama8b", choices=["llama8b", "cfg0", "small", "mixed", "streamed", "hooked"])
     ap.add_argument("--layers", type=int, default=32, help="transformer layers of the Llama-shaped set")
     ap.add_argument("--stream-gb", type=float, default=48.2, help="upper bound on pinned host bytes (streamed)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -218,7 +222,7 @@ def main() -> int:
         state_dtype = torch.bfloat16
         opt_kw.update(loss_scale=1024.0, max_grad_norm=1.0)
         bytes_per_elem = 24
-    else:  # streamed
+    else:  # streamed / hooked
         shapes = llama3_8b_shapes(args.layers)
         budget = int(args.stream_gb * 1e9)
         kept, used = [], 0
@@ -236,13 +240,15 @@ def main() -> int:
         state_dtype = torch.bfloat16
         opt_kw = dict(storage_device="cpu", seed=1234, stream_chunk_bytes=256 << 20)
         bytes_per_elem = 12
+        if wl == "hooked":
+            gmap_needed = False
 
     total = sum(numel(s) for s in shapes)
     opt = ramtorch_amd.AdamW(params, dtype=state_dtype, **HP, **opt_kw)
     for i, p in enumerate(params):
         st = opt.state[p]
         st["step"] = first_step - 1 - args.warmup
-        if wl != "streamed":
+        if wl not in ("streamed", "hooked"):
             st["ema"] = fill_tensor(p.shape, "m", 1234 + 4 * i + 2, torch.bfloat16, dev)
             vdt = torch.float32 if wl == "mixed" else torch.bfloat16
             st["ema_squared"] = fill_tensor(p.shape, "v", 1234 + 4 * i + 3, vdt, dev)
@@ -257,12 +263,23 @@ def main() -> int:
     torch.cuda.synchronize()
 
     handle = adamw_mod._handle(0)
+    if "RT_MAX_INFLIGHT_BYTES" in os.environ:  # experiment knob: gradient bytes step_param may keep alive
+        opt.max_inflight_bytes = int(os.environ["RT_MAX_INFLIGHT_BYTES"])
+
+    def one_step():
+        if wl == "hooked":
+            for p, g in zip(reversed(params), reversed(grads)):
+                opt.step_param(p, g)
+            opt.step()
+        else:
+            opt.step(noise=noise, grads=gmap)
+
     for _ in range(args.warmup):
-        opt.step(noise=noise, grads=gmap)
+        one_step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        opt.step(noise=noise, grads=gmap)
+        one_step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
@@ -271,7 +288,7 @@ def main() -> int:
     # that reading the events does not serialise the timed region above)
     roofline = None
     stream_info = None
-    if wl != "streamed":
+    if wl not in ("streamed", "hooked"):
         handle.set_timing(True)
         ks = []
         for _ in range(min(args.steps, 10)):
@@ -297,7 +314,10 @@ def main() -> int:
         roofline["frac_of_pattern_ceiling"] = achieved / roofline["pattern_ceiling_GBps"] if wl in ("llama8b", "small") else None
         del bufs
     else:
-        st = handle.streamed_stats()
+        if wl == "streamed":
+            st = handle.streamed_stats()
+        else:  # per-tensor asynchronous calls: the whole step is the unit
+            st = {"bytes_h2d": 6.0 * total, "bytes_d2h": 6.0 * total, "seconds": ms_per_step * 1e-3}
         stream_info = {"h2d_GBps": st["bytes_h2d"] / st["seconds"] / 1e9, "d2h_GBps": st["bytes_d2h"] / st["seconds"] / 1e9,
                        "seconds_last_call": st["seconds"], "host_bytes": 6 * total}
         # same-run pinned-copy peaks with the same chunk size

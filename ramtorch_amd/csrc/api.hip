@@ -11,6 +11,7 @@
 #include <deque>
 #include <map>
 #include <new>
+#include <thread>
 #include <vector>
 
 #include "kernels.h"
@@ -69,16 +70,20 @@ struct Streamed {
     hipEvent_t comp_done[2] = {nullptr, nullptr};
     hipEvent_t d2h_done[2] = {nullptr, nullptr};
     DevBuf stage[4][2];  // [p,g,m,v][buffer]
-    // Table images of every chunk of one call, back to back.  A small ring, because an
-    // asynchronous call may still be running when the next one builds its tables.
+    // Table images of every chunk of one call, back to back.  A pool, because an
+    // asynchronous call may still be running when the next one builds its tables; a
+    // free entry is found by polling and the pool grows when there is none.  The host
+    // never blocks here: a host thread waiting on an event while the copy pipeline is
+    // running was measured to cut the copy rate by a third (the runtime resolves the
+    // cross-stream dependencies of the copies on the host).
     struct TableRing {
         DevBuf dev;
         void* host = nullptr;  // pinned image
         size_t host_cap = 0;
         hipEvent_t done = nullptr;  // recorded after the last kernel that reads `dev`
         bool in_flight = false;
-    } ring[4];
-    uint32_t ring_pos = 0;
+    };
+    std::vector<TableRing> ring;
     // The pipeline state survives across calls so that asynchronous calls chain correctly:
     uint64_t seq = 0;                      // chunks enqueued so far; chunk `seq` uses buffer seq & 1
     bool used_buf[2] = {false, false};     // buffer has a D2H whose completion the next H2D must await
@@ -626,7 +631,6 @@ static int streamed_init(rt_handle* h) {
         HIP_TRY(hipEventCreateWithFlags(&st.comp_done[b], hipEventDisableTiming));
         HIP_TRY(hipEventCreateWithFlags(&st.d2h_done[b], hipEventDisableTiming));
     }
-    for (auto& r : st.ring) HIP_TRY(hipEventCreateWithFlags(&r.done, hipEventDisableTiming));
     st.ready = true;
     return RT_OK;
 }
@@ -703,6 +707,15 @@ static int streamed_wait(rt_handle* h) {
     Streamed& st = h->st;
     if (!st.ready) return RT_OK;
     HIP_TRY(hipSetDevice(h->device));
+    // Sleep-poll until the last ticket has landed, then synchronise (which returns at once).
+    // A host thread spinning inside the runtime while the pipeline runs slows the copies
+    // down: the runtime resolves their cross-stream dependencies on host threads.
+    while (!st.ticket_events.empty()) {
+        hipError_t q = hipEventQuery(st.ticket_events.back().second);
+        if (q == hipSuccess) break;
+        if (q != hipErrorNotReady) return fail(RT_EHIP, "hipEventQuery failed: %s", hipGetErrorString(q));
+        std::this_thread::sleep_for(std::chrono::microseconds(200));
+    }
     HIP_TRY(hipStreamSynchronize(st.d2h));
     HIP_TRY(hipStreamSynchronize(st.comp));
     HIP_TRY(hipStreamSynchronize(st.h2d));
@@ -799,11 +812,23 @@ static int streamed_enqueue(rt_handle* h, const rt_tensor_desc* descs, uint32_t 
         blob.resize(plan_off[c] + plans[c].bytes);
         if (plans[c].bytes) memcpy(blob.data() + plan_off[c], h->image.data(), plans[c].bytes);
     }
-    Streamed::TableRing& tab = st.ring[st.ring_pos++ % 4];
-    if (tab.in_flight) {
-        HIP_TRY(hipEventSynchronize(tab.done));
-        tab.in_flight = false;
+    size_t slot = st.ring.size();
+    for (size_t i = 0; i < st.ring.size(); ++i) {
+        if (st.ring[i].in_flight) {
+            hipError_t q = hipEventQuery(st.ring[i].done);
+            if (q == hipSuccess) st.ring[i].in_flight = false;
+            else if (q != hipErrorNotReady) return fail(RT_EHIP, "hipEventQuery failed: %s", hipGetErrorString(q));
+        }
+        if (!st.ring[i].in_flight) {
+            slot = i;
+            break;
+        }
     }
+    if (slot == st.ring.size()) {
+        st.ring.emplace_back();
+        HIP_TRY(hipEventCreateWithFlags(&st.ring.back().done, hipEventDisableTiming));
+    }
+    Streamed::TableRing& tab = st.ring[slot];
     if (blob.size() > tab.host_cap) {
         if (tab.host) HIP_TRY(hipHostFree(tab.host));
         tab.host = nullptr;
@@ -813,7 +838,7 @@ static int streamed_enqueue(rt_handle* h, const rt_tensor_desc* descs, uint32_t 
         if (e != hipSuccess) return fail(RT_ENOMEM, "hipHostMalloc(%zu) failed: %s", want, hipGetErrorString(e));
         tab.host_cap = want;
     }
-    rc = dev_reserve(tab.dev, blob.size());
+    rc = dev_reserve(tab.dev, blob.size() + 16);
     if (rc != RT_OK) return rc;
     memcpy(tab.host, blob.data(), blob.size());
 
@@ -821,8 +846,13 @@ static int streamed_enqueue(rt_handle* h, const rt_tensor_desc* descs, uint32_t 
     HIP_TRY(hipEventRecord(st.start, user));
     HIP_TRY(hipStreamWaitEvent(st.h2d, st.start, 0));
     HIP_TRY(hipStreamWaitEvent(st.comp, st.start, 0));
-    if (!blob.empty())
-        HIP_TRY(hipMemcpyAsync(tab.dev.ptr, tab.host, blob.size(), hipMemcpyHostToDevice, st.comp));
+    if (!blob.empty()) {
+        const uint64_t n_vec = (blob.size() + 15) / 16;  // buffers are padded well past the blob
+        const uint32_t grid = (uint32_t)std::min<uint64_t>((n_vec + kThreads - 1) / kThreads, 64);
+        hipLaunchKernelGGL(table_upload_kernel, dim3(grid), dim3(kThreads), 0, st.comp, (uint64_t)tab.dev.ptr,
+                           (uint64_t)tab.host, n_vec);
+        HIP_TRY(hipGetLastError());
+    }
 
     st.bytes_h2d = st.bytes_d2h = 0;
     st.timeline.clear();

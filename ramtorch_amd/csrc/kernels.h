@@ -412,6 +412,17 @@ __global__ __launch_bounds__(kThreads) void sr_adamw_generic_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// Copies a table image from pinned host memory (read over the host link by the
+// kernel itself) into device memory.  The streamed pipeline uses this instead
+// of a DMA copy: a small hipMemcpyAsync queued between the large H2D / D2H
+// copies was measured to slow the D2H copies down fourfold.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void table_upload_kernel(uint64_t dst, uint64_t src_host, uint64_t n_vec) {
+    for (uint64_t i = (uint64_t)blockIdx.x * kThreads + threadIdx.x; i < n_vec; i += (uint64_t)gridDim.x * kThreads)
+        *(RT_GLOBAL u32x4*)(dst + i * 16) = *(const RT_GLOBAL u32x4*)(src_host + i * 16);
+}
+
+// ---------------------------------------------------------------------------
 // Stream probe: the memory traffic of the all-bf16 fast kernel (read p, g, m, v;
 // write p, m, v in place, same chunking and prefetch) with the arithmetic
 // replaced by two integer ops.  Its rate is what this access pattern can get

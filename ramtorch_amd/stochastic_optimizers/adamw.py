@@ -9,6 +9,7 @@ There is no CPU or eager fallback: ``step()`` needs the HIP library and a GPU.
 """
 from __future__ import annotations
 
+import time
 from typing import Dict, List, Optional
 
 import numpy as np
@@ -114,6 +115,7 @@ class AdamW(Optimizer):
         self.max_inflight_bytes = 2 << 30  # gradients kept alive for updates still in flight (step_param)
         self._stepped_early = set()       # id(param) updated by step_param since the last step()
         self._inflight = []               # (device, ticket, bytes, tensors kept alive)
+        self._early_batch = {}            # device -> [[entry, scalars, handed-over elements], ...], pending elements
         # eager state allocation, as adamw.py:84-104
         for group in self.param_groups:
             for p in group["params"]:
@@ -447,12 +449,60 @@ class AdamW(Optimizer):
                 if e.p.is_cuda and e.m.is_cuda and e.v.is_cuda:
                     F.step_resident(h, [e], sc, seed=self.seed, explicit_noise=False)  # stream-ordered already
                 else:
-                    chunk_elems = max(8, (self.stream_chunk_bytes // 2) // 8 * 8)
-                    ticket = F.step_streamed(h, [e], sc, seed=self.seed, explicit_noise=False,
-                                             chunk_elems=chunk_elems, wait=False)
-                    self._inflight.append((dev, ticket, g.numel() * g.element_size(), (g, e)))
-                    self._release_finished(dev)
+                    # Tensors are handed to the copy pipeline in pieces of exactly one staging chunk
+                    # (a tensor may be cut, at a multiple of 8 elements): chunks of equal size keep
+                    # H2D and D2H overlapped, a run of unequal tensors would not.
+                    batch = self._early_batch.setdefault(dev, [[], 0])
+                    batch[0].append([e, sc[0], 0])      # entry, its scalars, elements already handed over
+                    batch[1] += e.p.numel()
+                    self._flush_early_batch(dev, final=False)
         self._stepped_early.add(id(p))
+
+    def _flush_early_batch(self, dev: int, final: bool) -> None:
+        batch = self._early_batch.get(dev)
+        if not batch:
+            return
+        chunk_elems = max(8, (self.stream_chunk_bytes // 2) // 8 * 8)
+        h = _handle(dev)
+        while batch[0] and (batch[1] >= chunk_elems or final):
+            room = chunk_elems
+            entries, scalars = [], []
+            while batch[0] and room >= 8:
+                item = batch[0][0]
+                e, sc, used = item
+                n = e.p.numel()
+                take = min(n - used, room)
+                if take < n - used:
+                    take -= take % 8            # a cut must fall on a Philox block boundary
+                    if take == 0:
+                        break
+                if used == 0 and take == n:
+                    piece = e
+                else:
+                    sl = slice(used, used + take)
+                    piece = F.Entry(p=e.p.view(-1)[sl], g=e.g.view(-1)[sl], m=e.m.view(-1)[sl], v=e.v.view(-1)[sl],
+                                    step=e.step, scalars_idx=0, tensor_id=e.tensor_id,
+                                    elem_offset=e.elem_offset + used, keep=[e])
+                piece.scalars_idx = len(scalars)
+                scalars.append(sc)
+                entries.append(piece)
+                room -= take
+                room -= room % 8                # the next piece starts 16-byte aligned in staging
+                batch[1] -= take
+                if used + take == n:
+                    batch[0].pop(0)
+                else:
+                    item[2] = used + take
+            if not entries:
+                break
+            with torch.cuda.device(dev):
+                ticket = F.step_streamed(h, entries, scalars, seed=self.seed, explicit_noise=False,
+                                         chunk_elems=chunk_elems, wait=False)
+            nbytes = sum(x.g.numel() * x.g.element_size() for x in entries)
+            self._inflight.append((dev, ticket, nbytes, entries))
+            self._release_finished(dev)
+        if not batch[0]:
+            self._early_batch.pop(dev, None)
 
     def _release_finished(self, dev: int) -> None:
         """Drop the references of finished asynchronous updates; if too many gradient bytes
@@ -461,11 +511,17 @@ class AdamW(Optimizer):
         done = h.streamed_completed()
         self._inflight = [x for x in self._inflight if not (x[0] == dev and x[1] <= done)]
         if sum(x[2] for x in self._inflight) > self.max_inflight_bytes:
-            h.streamed_wait()
-            self._inflight = [x for x in self._inflight if x[0] != dev]
+            # Let the oldest updates finish, polling with short sleeps: a host thread that
+            # blocks inside the runtime while the copy pipeline runs slows the copies down.
+            while sum(x[2] for x in self._inflight) > self.max_inflight_bytes // 2:
+                time.sleep(0.0005)
+                done = h.streamed_completed()
+                self._inflight = [x for x in self._inflight if not (x[0] == dev and x[1] <= done)]
 
     def finish_early_steps(self) -> None:
         """Wait until every update started by ``step_param`` has landed in host memory."""
+        for dev in list(self._early_batch):
+            self._flush_early_batch(dev, final=True)
         for dev in sorted({x[0] for x in self._inflight}):
             with torch.cuda.device(dev):
                 _handle(dev).streamed_wait()
