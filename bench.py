@@ -263,8 +263,10 @@ def main() -> int:
     torch.cuda.synchronize()
 
     handle = adamw_mod._handle(0)
-    if "RT_MAX_INFLIGHT_BYTES" in os.environ:  # experiment knob: gradient bytes step_param may keep alive
-        opt.max_inflight_bytes = int(os.environ["RT_MAX_INFLIGHT_BYTES"])
+    if "RT_MAX_INFLIGHT_CALLS" in os.environ:  # experiment knob: chunks step_param may queue ahead
+        opt.max_inflight_calls = int(os.environ["RT_MAX_INFLIGHT_CALLS"])
+    if "RT_POLL_SECONDS" in os.environ:
+        opt._poll_seconds = float(os.environ["RT_POLL_SECONDS"])
 
     def one_step():
         if wl == "hooked":
@@ -333,6 +335,19 @@ def main() -> int:
             torch.cuda.synchronize()
             stream_info[f"pinned_{name}_peak_GBps"] = 8 * chunk / (time.perf_counter() - t1) / 1e9
         stream_info["h2d_frac_of_peak"] = stream_info["h2d_GBps"] / stream_info["pinned_h2d_peak_GBps"]
+        if wl == "streamed":
+            # per-chunk copy durations of one more step, from events the library records on its copy streams
+            handle.set_timing(True)
+            one_step()
+            tl = handle.streamed_timeline()
+            handle.set_timing(False)
+            if tl:
+                h2d = [r[1] - r[0] for r in tl]
+                d2h = [r[3] - r[2] for r in tl]
+                stream_info["chunks"] = len(tl)
+                stream_info["h2d_chunk_ms"] = {"first": h2d[0], "median": sorted(h2d)[len(h2d) // 2], "max": max(h2d)}
+                stream_info["d2h_chunk_ms"] = {"median": sorted(d2h)[len(d2h) // 2], "max": max(d2h), "last": d2h[-1]}
+                stream_info["pipeline_ms"] = tl[-1][3] - tl[0][0]
         roofline = {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": None,
                     "traffic": None, "note": "host-link bound; see host_link"}
 

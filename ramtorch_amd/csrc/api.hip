@@ -45,6 +45,8 @@ static int fail(int code, const char* fmt, ...) {
 namespace {
 
 constexpr int kSlots = 2;            // table staging slots (host runs at most this far ahead)
+constexpr size_t kTablePool = 8;     // table images of streamed calls in flight
+constexpr size_t kTablePoolBytes = 64 << 10;
 constexpr int kNormPartials = 2048;  // workgroups of the norm pass
 
 struct DevBuf {
@@ -71,16 +73,15 @@ struct Streamed {
     hipEvent_t d2h_done[2] = {nullptr, nullptr};
     DevBuf stage[4][2];  // [p,g,m,v][buffer]
     // Table images of every chunk of one call, back to back.  A pool, because an
-    // asynchronous call may still be running when the next one builds its tables; a
-    // free entry is found by polling and the pool grows when there is none.  The host
-    // never blocks here: a host thread waiting on an event while the copy pipeline is
-    // running was measured to cut the copy rate by a third (the runtime resolves the
-    // cross-stream dependencies of the copies on the host).
+    // asynchronous call may still be running when the next one builds its tables; an
+    // entry is free again once the ticket of the call that used it has been published,
+    // and the pool grows when there is none.  The host never waits inside the runtime
+    // here (see streamed_wait).
     struct TableRing {
         DevBuf dev;
         void* host = nullptr;  // pinned image
         size_t host_cap = 0;
-        hipEvent_t done = nullptr;  // recorded after the last kernel that reads `dev`
+        uint64_t ticket = 0;  // call that reads `dev`; free again once that ticket is published
         bool in_flight = false;
     };
     std::vector<TableRing> ring;
@@ -88,9 +89,10 @@ struct Streamed {
     uint64_t seq = 0;                      // chunks enqueued so far; chunk `seq` uses buffer seq & 1
     bool used_buf[2] = {false, false};     // buffer has a D2H whose completion the next H2D must await
     bool pending = false;                  // work enqueued since the last wait
-    uint64_t tickets_issued = 0, tickets_done = 0;
-    std::deque<std::pair<uint64_t, hipEvent_t>> ticket_events;  // (ticket, recorded on d2h after its last copy)
-    std::vector<hipEvent_t> event_pool;
+    // Tickets: a one-thread kernel behind the last D2H copy of a call writes the call's number
+    // into a word of pinned host memory; the host learns about completion by reading that word.
+    uint64_t tickets_issued = 0;
+    volatile uint64_t* ticket_word = nullptr;
     bool ready = false;
     double bytes_h2d = 0, bytes_d2h = 0, seconds = 0;
     std::vector<hipEvent_t> tl_events;  // 4 per chunk when timing is on: H2D begin/end, D2H begin/end
@@ -465,10 +467,8 @@ int rt_destroy(rt_handle* h) {
     for (auto& r : st.ring) {
         if (r.dev.ptr) (void)hipFree(r.dev.ptr);
         if (r.host) (void)hipHostFree(r.host);
-        if (r.done) (void)hipEventDestroy(r.done);
     }
-    for (auto& te : st.ticket_events) (void)hipEventDestroy(te.second);
-    for (hipEvent_t e : st.event_pool) (void)hipEventDestroy(e);
+    if (st.ticket_word) (void)hipHostFree((void*)st.ticket_word);
     for (hipEvent_t e : st.tl_events) (void)hipEventDestroy(e);
     if (st.start) (void)hipEventDestroy(st.start);
     if (st.h2d) (void)hipStreamDestroy(st.h2d);
@@ -631,6 +631,20 @@ static int streamed_init(rt_handle* h) {
         HIP_TRY(hipEventCreateWithFlags(&st.comp_done[b], hipEventDisableTiming));
         HIP_TRY(hipEventCreateWithFlags(&st.d2h_done[b], hipEventDisableTiming));
     }
+    // Table memory for the calls in flight is set aside now: allocating (device or pinned
+    // host memory) while the copy pipeline runs stalls the copies for tens of milliseconds.
+    st.ring.resize(kTablePool);
+    for (auto& r : st.ring) {
+        int rc = dev_reserve(r.dev, kTablePoolBytes);
+        if (rc != RT_OK) return rc;
+        hipError_t e = hipHostMalloc(&r.host, kTablePoolBytes, hipHostMallocDefault);
+        if (e != hipSuccess) return fail(RT_ENOMEM, "hipHostMalloc(%zu) failed: %s", kTablePoolBytes, hipGetErrorString(e));
+        r.host_cap = kTablePoolBytes;
+    }
+    void* word = nullptr;
+    HIP_TRY(hipHostMalloc(&word, 64, hipHostMallocDefault));
+    *(volatile uint64_t*)word = 0;
+    st.ticket_word = (volatile uint64_t*)word;
     st.ready = true;
     return RT_OK;
 }
@@ -690,38 +704,26 @@ int rt_streamed_plan(const rt_tensor_desc* descs, uint32_t n, uint64_t chunk_ele
     return RT_OK;
 }
 
-// Retires finished tickets (non-blocking).
-static int streamed_poll(Streamed& st) {
-    while (!st.ticket_events.empty()) {
-        hipError_t e = hipEventQuery(st.ticket_events.front().second);
-        if (e == hipErrorNotReady) break;
-        if (e != hipSuccess) return fail(RT_EHIP, "hipEventQuery failed: %s", hipGetErrorString(e));
-        st.tickets_done = st.ticket_events.front().first;
-        st.event_pool.push_back(st.ticket_events.front().second);
-        st.ticket_events.pop_front();
-    }
-    return RT_OK;
+// Highest ticket whose copies have all landed: a plain read of pinned host memory.
+static inline uint64_t tickets_done(const Streamed& st) {
+    return st.ticket_word ? __atomic_load_n((const uint64_t*)st.ticket_word, __ATOMIC_ACQUIRE) : 0;
 }
 
 static int streamed_wait(rt_handle* h) {
     Streamed& st = h->st;
     if (!st.ready) return RT_OK;
     HIP_TRY(hipSetDevice(h->device));
-    // Sleep-poll until the last ticket has landed, then synchronise (which returns at once).
-    // A host thread spinning inside the runtime while the pipeline runs slows the copies
-    // down: the runtime resolves their cross-stream dependencies on host threads.
-    while (!st.ticket_events.empty()) {
-        hipError_t q = hipEventQuery(st.ticket_events.back().second);
-        if (q == hipSuccess) break;
-        if (q != hipErrorNotReady) return fail(RT_EHIP, "hipEventQuery failed: %s", hipGetErrorString(q));
-        std::this_thread::sleep_for(std::chrono::microseconds(200));
-    }
+    // Sleep until the last ticket has been published, then synchronise (which returns at
+    // once).  While the pipeline runs the host stays out of the runtime: a thread spinning
+    // in a synchronise call, or polling events, was measured to slow the copies down
+    // severalfold (the runtime resolves their cross-stream dependencies on host threads).
+    while (tickets_done(st) < st.tickets_issued) std::this_thread::sleep_for(std::chrono::microseconds(100));
     HIP_TRY(hipStreamSynchronize(st.d2h));
     HIP_TRY(hipStreamSynchronize(st.comp));
     HIP_TRY(hipStreamSynchronize(st.h2d));
     st.pending = false;
     for (auto& r : st.ring) r.in_flight = false;
-    return streamed_poll(st);
+    return RT_OK;
 }
 
 // Validates and enqueues the whole pipeline of one call; does not wait for it.
@@ -812,21 +814,20 @@ static int streamed_enqueue(rt_handle* h, const rt_tensor_desc* descs, uint32_t 
         blob.resize(plan_off[c] + plans[c].bytes);
         if (plans[c].bytes) memcpy(blob.data() + plan_off[c], h->image.data(), plans[c].bytes);
     }
+    // A free pool entry (the call that used it has published its ticket), preferably one that is
+    // already large enough.  With every entry in use the host sleeps until the oldest call is
+    // done -- reading the ticket word, not waiting inside the runtime.
     size_t slot = st.ring.size();
-    for (size_t i = 0; i < st.ring.size(); ++i) {
-        if (st.ring[i].in_flight) {
-            hipError_t q = hipEventQuery(st.ring[i].done);
-            if (q == hipSuccess) st.ring[i].in_flight = false;
-            else if (q != hipErrorNotReady) return fail(RT_EHIP, "hipEventQuery failed: %s", hipGetErrorString(q));
+    for (;;) {
+        const uint64_t done_now = tickets_done(st);
+        for (size_t i = 0; i < st.ring.size(); ++i) {
+            Streamed::TableRing& r = st.ring[i];
+            if (r.in_flight && r.ticket <= done_now) r.in_flight = false;
+            if (!r.in_flight && (slot == st.ring.size() || (st.ring[slot].host_cap < blob.size() && r.host_cap >= blob.size())))
+                slot = i;
         }
-        if (!st.ring[i].in_flight) {
-            slot = i;
-            break;
-        }
-    }
-    if (slot == st.ring.size()) {
-        st.ring.emplace_back();
-        HIP_TRY(hipEventCreateWithFlags(&st.ring.back().done, hipEventDisableTiming));
+        if (slot != st.ring.size()) break;
+        std::this_thread::sleep_for(std::chrono::microseconds(100));
     }
     Streamed::TableRing& tab = st.ring[slot];
     if (blob.size() > tab.host_cap) {
@@ -917,19 +918,14 @@ static int streamed_enqueue(rt_handle* h, const rt_tensor_desc* descs, uint32_t 
         st.used_buf[b] = true;
     }
     st.seq += chunks.size();
-    HIP_TRY(hipEventRecord(tab.done, st.comp));
+    tab.ticket = st.tickets_issued + 1;
     tab.in_flight = true;
-    // ticket: completes when the last D2H of this call has landed (D2H follows compute, so
+    // ticket: published when the last D2H of this call has landed (D2H follows compute, so
     // device-resident arrays are final by then as well)
-    hipEvent_t te;
-    if (!st.event_pool.empty()) {
-        te = st.event_pool.back();
-        st.event_pool.pop_back();
-    } else {
-        HIP_TRY(hipEventCreateWithFlags(&te, hipEventDisableTiming));
-    }
-    HIP_TRY(hipEventRecord(te, st.d2h));
-    st.ticket_events.emplace_back(++st.tickets_issued, te);
+    ++st.tickets_issued;
+    hipLaunchKernelGGL(publish_ticket_kernel, dim3(1), dim3(1), 0, st.d2h, (uint64_t)st.ticket_word,
+                       st.tickets_issued);
+    HIP_TRY(hipGetLastError());
     if (ticket_out) *ticket_out = st.tickets_issued;
     if (trace) st.timeline.assign(4 * chunks.size(), 0.0f);
     return RT_OK;
@@ -967,9 +963,8 @@ int rt_streamed_wait(rt_handle* h) {
 
 int rt_streamed_completed(rt_handle* h, uint64_t* ticket_done) {
     if (!h || !ticket_done) return fail(RT_EINVAL, "NULL argument");
-    int rc = streamed_poll(h->st);
-    *ticket_done = h->st.tickets_done;
-    return rc;
+    *ticket_done = tickets_done(h->st);
+    return RT_OK;
 }
 
 

@@ -422,6 +422,13 @@ __global__ __launch_bounds__(kThreads) void table_upload_kernel(uint64_t dst, ui
         *(RT_GLOBAL u32x4*)(dst + i * 16) = *(const RT_GLOBAL u32x4*)(src_host + i * 16);
 }
 
+// Publishes a ticket number to a word in pinned host memory.  Queued on the D2H
+// stream behind the last copy of a call, it lets the host see completion by
+// reading memory, without entering the runtime.
+__global__ void publish_ticket_kernel(uint64_t host_word, uint64_t ticket) {
+    __hip_atomic_store((RT_GLOBAL uint64_t*)host_word, ticket, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // ---------------------------------------------------------------------------
 // Stream probe: the memory traffic of the all-bf16 fast kernel (read p, g, m, v;
 // write p, m, v in place, same chunking and prefetch) with the arithmetic

@@ -113,6 +113,8 @@ class AdamW(Optimizer):
         self.last_grad_norm: Optional[torch.Tensor] = None  # [norm, clip_coef, found_inf bits, -] on the GPU
         self.fuse_in_backward = True      # the hook of make_post_accumulate_hook() is live
         self.max_inflight_bytes = 2 << 30  # gradients kept alive for updates still in flight (step_param)
+        self.max_inflight_calls = 2       # staging chunks handed to the copy pipeline and not finished yet
+        self._poll_seconds = 0.0002       # completion is read from host memory; no runtime call while waiting
         self._stepped_early = set()       # id(param) updated by step_param since the last step()
         self._inflight = []               # (device, ticket, bytes, tensors kept alive)
         self._early_batch = {}            # device -> [[entry, scalars, handed-over elements], ...], pending elements
@@ -495,28 +497,30 @@ class AdamW(Optimizer):
                     item[2] = used + take
             if not entries:
                 break
+            self._wait_for_room(dev)
             with torch.cuda.device(dev):
                 ticket = F.step_streamed(h, entries, scalars, seed=self.seed, explicit_noise=False,
                                          chunk_elems=chunk_elems, wait=False)
             nbytes = sum(x.g.numel() * x.g.element_size() for x in entries)
             self._inflight.append((dev, ticket, nbytes, entries))
-            self._release_finished(dev)
         if not batch[0]:
             self._early_batch.pop(dev, None)
 
-    def _release_finished(self, dev: int) -> None:
-        """Drop the references of finished asynchronous updates; if too many gradient bytes
-        are still held, wait for the pipeline."""
+    def _wait_for_room(self, dev: int) -> None:
+        """Drop the references of finished asynchronous updates and wait until fewer than
+        ``max_inflight_calls`` chunks are in flight.  Two chunks keep both staging buffers
+        busy (the next H2D overlaps the previous D2H); on the test machine a third chunk
+        queued while two are running made individual copies four times slower.  Completion
+        is a number the pipeline writes into pinned host memory, so waiting for it never
+        enters the runtime."""
         h = _handle(dev)
-        done = h.streamed_completed()
-        self._inflight = [x for x in self._inflight if not (x[0] == dev and x[1] <= done)]
-        if sum(x[2] for x in self._inflight) > self.max_inflight_bytes:
-            # Let the oldest updates finish, polling with short sleeps: a host thread that
-            # blocks inside the runtime while the copy pipeline runs slows the copies down.
-            while sum(x[2] for x in self._inflight) > self.max_inflight_bytes // 2:
-                time.sleep(0.0005)
-                done = h.streamed_completed()
-                self._inflight = [x for x in self._inflight if not (x[0] == dev and x[1] <= done)]
+        while True:
+            done = h.streamed_completed()
+            self._inflight = [x for x in self._inflight if not (x[0] == dev and x[1] <= done)]
+            mine = [x for x in self._inflight if x[0] == dev]
+            if len(mine) < self.max_inflight_calls and sum(x[2] for x in mine) <= self.max_inflight_bytes:
+                return
+            time.sleep(self._poll_seconds)
 
     def finish_early_steps(self) -> None:
         """Wait until every update started by ``step_param`` has landed in host memory."""
