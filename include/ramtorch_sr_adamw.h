@@ -31,7 +31,8 @@ extern "C" {
 /* element types */
 #define RT_DT_BF16 0
 #define RT_DT_F32 1
-#define RT_DT_F16 2 /* gradients only */
+#define RT_DT_F16 2
+#define RT_DT_F64 3 /* params and states only */
 
 /* where the rounding noise comes from */
 #define RT_NOISE_PHILOX 0   /* Philox4x32-10 keyed by seed; counter from (step, tensor, element) */
@@ -86,10 +87,10 @@ typedef struct rt_tensor_desc {
     uint32_t tensor_id;    /* < 2^30; part of the Philox counter */
     uint32_t step;         /* state["step"] after the increment (adamw.py:177), mod 2^32 */
     uint32_t scalars_idx;  /* index into the rt_scalars array */
-    uint8_t p_dtype;       /* RT_DT_BF16 (stochastic rounding) or RT_DT_F32 (plain store) */
+    uint8_t p_dtype;       /* RT_DT_BF16 (stochastic rounding); RT_DT_F32 / F16 / F64 (plain copy_, round to nearest) */
     uint8_t g_dtype;       /* RT_DT_BF16, RT_DT_F32 or RT_DT_F16 */
-    uint8_t m_dtype;       /* RT_DT_BF16 or RT_DT_F32 */
-    uint8_t v_dtype;       /* RT_DT_BF16 or RT_DT_F32 */
+    uint8_t m_dtype;       /* as p_dtype */
+    uint8_t v_dtype;       /* as p_dtype */
     uint32_t host_mask;    /* RT_HOST_* bits; must be 0 for rt_step_multi */
     uint32_t reserved;
 } rt_tensor_desc;

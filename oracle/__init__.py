@@ -31,10 +31,11 @@ ADDCDIV_AM_FIRST = 32
 TORCH_CPU_FLAVOUR = FMA_ADD | FMA_ADDCMUL | ADDCMUL_AG_FIRST | ADDCDIV_AM_FIRST
 #: rounding sequence of torch's GPU (ROCm) kernels -- what the reference executes,
 #: since adamw.py:152-157 always computes on a GPU.  Pinned on the GPU box by
-#: tests/test_flavour_gpu.py against the ATen kernels themselves.
+#: tests/test_gpu_parity.py against the ATen kernels themselves, and here by the
+#: golden vectors those kernels produced (tests/golden/torch_gpu_step.npz).
 REFERENCE_FLAVOUR = FMA_ADD | FMA_ADDCMUL | FMA_ADDCDIV | DIV_RECIP
 
-DT_BF16, DT_F32, DT_F16 = 0, 1, 2
+DT_BF16, DT_F32, DT_F16, DT_F64 = 0, 1, 2, 3
 NOISE_PHILOX, NOISE_EXPLICIT = 0, 1
 
 
@@ -79,6 +80,10 @@ def lib() -> ctypes.CDLL:
         L.orc_bf16_to_f32.argtypes = [ctypes.c_uint16]
         L.orc_f16_to_f32.restype = ctypes.c_float
         L.orc_f16_to_f32.argtypes = [ctypes.c_uint16]
+        L.orc_f32_to_f16_rne.restype = ctypes.c_uint16
+        L.orc_f32_to_f16_rne.argtypes = [ctypes.c_float]
+        L.orc_f32_to_f16_array.restype = None
+        L.orc_f32_to_f16_array.argtypes = [f32p, u16p, ctypes.c_uint64]
         L.orc_philox4x32_10.restype = None
         L.orc_philox4x32_10.argtypes = [ctypes.POINTER(ctypes.c_uint32)] * 3
         L.orc_philox_noise.restype = ctypes.c_uint16
@@ -128,7 +133,7 @@ def scalars_from_hparams(lr, betas, eps, weight_decay, step, inv_loss_scale=1.0,
     )
 
 
-_NP_DT = {DT_BF16: np.uint16, DT_F16: np.uint16, DT_F32: np.float32}
+_NP_DT = {DT_BF16: np.uint16, DT_F16: np.uint16, DT_F32: np.float32, DT_F64: np.float64}
 
 
 def _ptr(a, ctype):
@@ -236,6 +241,14 @@ def f32_to_bf16_rne(x: np.ndarray) -> np.ndarray:
     b = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
     r = ((b + 0x7FFF + ((b >> 16) & 1)) >> 16).astype(np.uint16)
     return r
+
+
+def f32_to_f16_rne(x: np.ndarray) -> np.ndarray:
+    """The oracle's float32 -> binary16 conversion (bits), for fp16 params / states."""
+    x = np.ascontiguousarray(x, np.float32).ravel()
+    out = np.empty(x.size, np.uint16)
+    lib().orc_f32_to_f16_array(_ptr(x, ctypes.c_float), _ptr(out, ctypes.c_uint16), x.size)
+    return out
 
 
 def bf16_to_f32(h: np.ndarray) -> np.ndarray:

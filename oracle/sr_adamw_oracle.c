@@ -35,6 +35,7 @@
 #define ORC_DT_BF16 0
 #define ORC_DT_F32 1
 #define ORC_DT_F16 2
+#define ORC_DT_F64 3
 
 #define ORC_NOISE_PHILOX 0
 #define ORC_NOISE_EXPLICIT 1
@@ -83,6 +84,42 @@ float orc_f16_to_f32(uint16_t h) {
     }
     if (exp == 31) return bits_to_f32(sign | 0x7F800000u | (man << 13));
     return bits_to_f32(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+/*
+ * fp32 -> IEEE binary16, round to nearest even with gradual underflow: the
+ * conversion Tensor.copy_ performs when a param or state is kept in fp16
+ * (adamw.py:208,214,221-222).  NaN payloads are not part of the contract
+ * (a quiet NaN of the same sign is returned).
+ */
+uint16_t orc_f32_to_f16_rne(float x) {
+    uint32_t b = f32_to_bits(x);
+    uint16_t sign = (uint16_t)((b >> 16) & 0x8000u);
+    uint32_t a = b & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return (uint16_t)(sign | 0x7E00u);
+    if (a == 0x7F800000u) return (uint16_t)(sign | 0x7C00u);
+    int32_t exp = (int32_t)(a >> 23) - 127 + 15; /* biased binary16 exponent */
+    uint32_t man = a & 0x7FFFFFu;
+    if (exp >= 31) return (uint16_t)(sign | 0x7C00u);
+    if (exp <= 0) {
+        /* subnormal result: the 24-bit significand moves right by 14 - exp */
+        int32_t shift = 14 - exp;
+        if (shift > 25 || a == 0) return sign;
+        uint32_t sig = man | 0x800000u;
+        uint32_t half = sig >> shift;
+        uint32_t rem = sig & ((1u << shift) - 1u);
+        uint32_t mid = 1u << (shift - 1);
+        if (rem > mid || (rem == mid && (half & 1u))) ++half;
+        return (uint16_t)(sign | half);
+    }
+    uint32_t half = ((uint32_t)exp << 10) | (man >> 13);
+    uint32_t rem = man & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (half & 1u))) ++half; /* may carry up to infinity */
+    return (uint16_t)(sign | half);
+}
+
+void orc_f32_to_f16_array(const float* x, uint16_t* out, uint64_t n) {
+    for (uint64_t i = 0; i < n; ++i) out[i] = orc_f32_to_f16_rne(x[i]);
 }
 
 /*
@@ -216,14 +253,26 @@ static inline float load_as_f32(const void* base, int dtype, uint64_t i) {
     switch (dtype) {
         case ORC_DT_BF16: return orc_bf16_to_f32(((const uint16_t*)base)[i]);
         case ORC_DT_F16: return orc_f16_to_f32(((const uint16_t*)base)[i]);
+        case ORC_DT_F64: return (float)((const double*)base)[i]; /* .to(float32): round to nearest even */
         default: return ((const float*)base)[i];
+    }
+}
+
+/* Write-back of one element of p / ema / ema_squared (adamw.py:204-222): bf16 is
+ * stochastically rounded, every other dtype takes a plain copy_ (round to nearest). */
+static inline void store_from_f32(void* base, int dtype, uint64_t i, float x, uint16_t noise) {
+    switch (dtype) {
+        case ORC_DT_BF16: ((uint16_t*)base)[i] = orc_sr_bf16(x, noise); break;
+        case ORC_DT_F16: ((uint16_t*)base)[i] = orc_f32_to_f16_rne(x); break;
+        case ORC_DT_F64: ((double*)base)[i] = (double)x; break;
+        default: ((float*)base)[i] = x; break;
     }
 }
 
 /*
  * Whole-tensor step: upcast (adamw.py:160-170), update (:190-200), write back
- * (:204-222: bf16 targets are stochastically rounded, fp32 targets are stored
- * as they are).  `elem_offset` is the index, within the logical tensor, of the
+ * (:204-222: bf16 targets are stochastically rounded, fp32 / fp16 / fp64 targets
+ * take a plain copy_).  `elem_offset` is the index, within the logical tensor, of the
  * first element passed in (a multiple of 8), so that a tensor processed in
  * pieces draws the same noise as one processed whole.  dbg_* (optional) get
  * the fp32 values before rounding.  Returns 0, or a negative argument error.
@@ -234,10 +283,8 @@ int orc_step_tensor(void* p, int p_dtype, const void* g, int g_dtype, void* m, i
                     const uint16_t* noise_v, uint64_t seed, uint32_t step, uint32_t tensor_id,
                     uint64_t elem_offset, uint32_t flavour, float* dbg_p, float* dbg_m,
                     float* dbg_v) {
-    if (p_dtype != ORC_DT_BF16 && p_dtype != ORC_DT_F32) return -1;
-    if (m_dtype != ORC_DT_BF16 && m_dtype != ORC_DT_F32) return -1;
-    if (v_dtype != ORC_DT_BF16 && v_dtype != ORC_DT_F32) return -1;
-    if (g_dtype < 0 || g_dtype > 2) return -1;
+    if (p_dtype < 0 || p_dtype > 3 || m_dtype < 0 || m_dtype > 3 || v_dtype < 0 || v_dtype > 3) return -1;
+    if (g_dtype < 0 || g_dtype > 3) return -1;
     if (elem_offset & 7u) return -2;
     if (noise_mode == ORC_NOISE_EXPLICIT) {
         if (p_dtype == ORC_DT_BF16 && !noise_p) return -3;
@@ -255,27 +302,16 @@ int orc_step_tensor(void* p, int p_dtype, const void* g, int g_dtype, void* m, i
         if (dbg_m) dbg_m[i] = mo;
         if (dbg_v) dbg_v[i] = vo;
         uint64_t e = elem_offset + i;
-        if (p_dtype == ORC_DT_BF16) {
-            uint16_t n = noise_mode == ORC_NOISE_EXPLICIT ? noise_p[i]
-                                                          : orc_philox_noise(seed, step, tensor_id, 0, e);
-            ((uint16_t*)p)[i] = orc_sr_bf16(po, n);
-        } else {
-            ((float*)p)[i] = po;
-        }
-        if (m_dtype == ORC_DT_BF16) {
-            uint16_t n = noise_mode == ORC_NOISE_EXPLICIT ? noise_m[i]
-                                                          : orc_philox_noise(seed, step, tensor_id, 1, e);
-            ((uint16_t*)m)[i] = orc_sr_bf16(mo, n);
-        } else {
-            ((float*)m)[i] = mo;
-        }
-        if (v_dtype == ORC_DT_BF16) {
-            uint16_t n = noise_mode == ORC_NOISE_EXPLICIT ? noise_v[i]
-                                                          : orc_philox_noise(seed, step, tensor_id, 2, e);
-            ((uint16_t*)v)[i] = orc_sr_bf16(vo, n);
-        } else {
-            ((float*)v)[i] = vo;
-        }
+        uint16_t np16 = 0, nm16 = 0, nv16 = 0;
+        if (p_dtype == ORC_DT_BF16)
+            np16 = noise_mode == ORC_NOISE_EXPLICIT ? noise_p[i] : orc_philox_noise(seed, step, tensor_id, 0, e);
+        if (m_dtype == ORC_DT_BF16)
+            nm16 = noise_mode == ORC_NOISE_EXPLICIT ? noise_m[i] : orc_philox_noise(seed, step, tensor_id, 1, e);
+        if (v_dtype == ORC_DT_BF16)
+            nv16 = noise_mode == ORC_NOISE_EXPLICIT ? noise_v[i] : orc_philox_noise(seed, step, tensor_id, 2, e);
+        store_from_f32(p, p_dtype, i, po, np16);
+        store_from_f32(m, m_dtype, i, mo, nm16);
+        store_from_f32(v, v_dtype, i, vo, nv16);
     }
     return 0;
 }

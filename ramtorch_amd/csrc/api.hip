@@ -7,8 +7,9 @@
 #include <chrono>
 #include <cstdarg>
 #include <cstdio>
+#include <climits>
+#include <cstdint>
 #include <cstring>
-#include <deque>
 #include <map>
 #include <new>
 #include <thread>
@@ -48,6 +49,7 @@ constexpr int kSlots = 2;            // table staging slots (host runs at most t
 constexpr size_t kTablePool = 8;     // table images of streamed calls in flight
 constexpr size_t kTablePoolBytes = 64 << 10;
 constexpr int kNormPartials = 2048;  // workgroups of the norm pass
+constexpr uint64_t kMaxGrid = 0x7FFFFFFFull;  // workgroups of one launch (one per chunk of 8192 elements)
 
 struct DevBuf {
     void* ptr = nullptr;
@@ -130,7 +132,7 @@ static int dev_reserve(DevBuf& b, size_t bytes) {
     return RT_OK;
 }
 
-static int dtype_size(int dt) { return dt == RT_DT_F32 ? 4 : 2; }
+static int dtype_size(int dt) { return dt == RT_DT_F32 ? 4 : dt == RT_DT_F64 ? 8 : 2; }
 
 // ---------------------------------------------------------------------------
 // kernel dispatch
@@ -169,9 +171,19 @@ static KernelPair pick_kernel(int p, int g, int m, int v, int noise) {
     return p == RT_DT_BF16 ? pick_g<RT_DT_BF16>(g, m, v, noise) : pick_g<RT_DT_F32>(g, m, v, noise);
 }
 
-static inline uint32_t combo_of(const rt_tensor_desc& d) {
+static inline uint32_t dtypes_of(const rt_tensor_desc& d) {
     return (uint32_t)d.p_dtype | ((uint32_t)d.g_dtype << 2) | ((uint32_t)d.m_dtype << 4) |
            ((uint32_t)d.v_dtype << 6);
+}
+
+// Tensors with an fp16 or fp64 param or state all go to the one runtime-typed kernel.
+constexpr uint32_t kComboAny = 0x100u;
+
+static inline bool compiled_pmv(int dt) { return dt == RT_DT_BF16 || dt == RT_DT_F32; }
+
+// Launch group of a tensor: its dtype combination when the templated kernels cover it.
+static inline uint32_t combo_of(const rt_tensor_desc& d) {
+    return (compiled_pmv(d.p_dtype) && compiled_pmv(d.m_dtype) && compiled_pmv(d.v_dtype)) ? dtypes_of(d) : kComboAny;
 }
 
 // ---------------------------------------------------------------------------
@@ -183,15 +195,13 @@ static int validate(const rt_tensor_desc* descs, uint32_t n, const rt_scalars* s
     if (n > 0 && (scalars == nullptr || n_scalars == 0)) return fail(RT_EINVAL, "scalars missing");
     if (noise_mode != RT_NOISE_PHILOX && noise_mode != RT_NOISE_EXPLICIT)
         return fail(RT_EINVAL, "unknown noise_mode %d", noise_mode);
+    uint64_t total_chunks = 0;
     for (uint32_t i = 0; i < n; ++i) {
         const rt_tensor_desc& d = descs[i];
-        if (d.p_dtype != RT_DT_BF16 && d.p_dtype != RT_DT_F32)
-            return fail(RT_EUNSUPPORTED, "tensor %u: p_dtype %d (need bf16 or f32)", i, d.p_dtype);
-        if (d.m_dtype != RT_DT_BF16 && d.m_dtype != RT_DT_F32)
-            return fail(RT_EUNSUPPORTED, "tensor %u: m_dtype %d (need bf16 or f32)", i, d.m_dtype);
-        if (d.v_dtype != RT_DT_BF16 && d.v_dtype != RT_DT_F32)
-            return fail(RT_EUNSUPPORTED, "tensor %u: v_dtype %d (need bf16 or f32)", i, d.v_dtype);
-        if (d.g_dtype > RT_DT_F16) return fail(RT_EINVAL, "tensor %u: g_dtype %d unknown", i, d.g_dtype);
+        if (d.p_dtype > RT_DT_F64 || d.m_dtype > RT_DT_F64 || d.v_dtype > RT_DT_F64)
+            return fail(RT_EINVAL, "tensor %u: unknown p/m/v dtype %d/%d/%d", i, d.p_dtype, d.m_dtype, d.v_dtype);
+        if (d.g_dtype > RT_DT_F16)
+            return fail(RT_EINVAL, "tensor %u: g_dtype %d (need bf16, f32 or f16)", i, d.g_dtype);
         if (d.scalars_idx >= n_scalars)
             return fail(RT_EINVAL, "tensor %u: scalars_idx %u >= %u", i, d.scalars_idx, n_scalars);
         if (d.tensor_id >= (1u << 30)) return fail(RT_EINVAL, "tensor %u: tensor_id %u >= 2^30", i, d.tensor_id);
@@ -207,6 +217,10 @@ static int validate(const rt_tensor_desc* descs, uint32_t n, const rt_scalars* s
             return fail(RT_EINVAL, "tensor %u: array pointer not aligned to its element size", i);
         if (d.numel / kChunkElems >= 0xFFFFFFFFull)
             return fail(RT_EUNSUPPORTED, "tensor %u: numel %llu too large", i, (unsigned long long)d.numel);
+        total_chunks += (d.numel + kChunkElems - 1) / kChunkElems;
+        if (total_chunks > kMaxGrid)
+            return fail(RT_EUNSUPPORTED, "more than %llu chunks of %u elements in one call",
+                        (unsigned long long)kMaxGrid, kChunkElems);
         if (noise_mode == RT_NOISE_EXPLICIT) {
             if ((d.p_dtype == RT_DT_BF16 && !d.noise_p) || (d.m_dtype == RT_DT_BF16 && !d.noise_m) ||
                 (d.v_dtype == RT_DT_BF16 && !d.noise_v))
@@ -283,6 +297,7 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
         t.row_len = d.row_len ? d.row_len : 1;
         t.tensor_id4 = d.tensor_id * 4u;
         t.set_idx = it->second;
+        t.dtypes = dtypes_of(d);
         const uint64_t all = t.p | t.g | t.m | t.v | t.np | t.nm | t.nv;
         t.flags = (all & 15u) == 0 ? kFlagAligned : 0u;
         total_chunks += (d.numel + kChunkElems - 1) / kChunkElems;
@@ -314,7 +329,7 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
         Batch b{combo, c, 0, 0, 0};
         auto n_whole = [&](size_t k) -> uint32_t {
             const DevTensor& t = tens[k];
-            const bool plain = (t.flags & kFlagAligned) && (t.dp | t.dm | t.dv | t.row_mean) == 0;
+            const bool plain = combo != kComboAny && (t.flags & kFlagAligned) && (t.dp | t.dm | t.dv | t.row_mean) == 0;
             return plain ? (uint32_t)(t.numel / kChunkElems) : 0u;
         };
         for (size_t k = k0; k < k1; ++k) {
@@ -374,8 +389,14 @@ static int enqueue_kernels(const Plan& plan, const uint8_t* base, uint64_t seed,
     const DevTensor* tens = (const DevTensor*)(base + plan.off_tensors);
     const ChunkRef* chunks = (const ChunkRef*)(base + plan.off_chunks);
     for (const Batch& b : plan.batches) {
-        const KernelPair k = pick_kernel(b.combo & 3, (b.combo >> 2) & 3, (b.combo >> 4) & 3, (b.combo >> 6) & 3,
-                                         noise_mode);
+        KernelPair k;
+        if (b.combo == kComboAny) {
+            k.fast = nullptr;  // n_fast is 0 for this group
+            k.generic = noise_mode == RT_NOISE_EXPLICIT ? sr_adamw_any_kernel<RT_NOISE_EXPLICIT>
+                                                        : sr_adamw_any_kernel<RT_NOISE_PHILOX>;
+        } else {
+            k = pick_kernel(b.combo & 3, (b.combo >> 2) & 3, (b.combo >> 4) & 3, (b.combo >> 6) & 3, noise_mode);
+        }
         if (b.n_fast) {
             hipLaunchKernelGGL(k.fast, dim3(b.n_fast), dim3(kThreads), 0, stream, tens, chunks + b.first_fast, sets,
                                (uint32_t)seed, (uint32_t)(seed >> 32), d_clip_coef, d_skip);
@@ -421,6 +442,8 @@ int rt_version(void) { return RT_ABI_VERSION; }
 
 const char* rt_last_error(void) { return g_err; }
 
+int rt_destroy(rt_handle* h);
+
 int rt_create(int device, rt_handle** out) {
     if (!out) return fail(RT_EINVAL, "out is NULL");
     *out = nullptr;
@@ -436,9 +459,15 @@ int rt_create(int device, rt_handle** out) {
     rt_handle* h = new (std::nothrow) rt_handle();
     if (!h) return fail(RT_ENOMEM, "out of host memory");
     h->device = device;
-    for (int i = 0; i < kSlots; ++i) HIP_TRY(hipEventCreateWithFlags(&h->slots[i].done, hipEventDisableTiming));
-    HIP_TRY(hipEventCreate(&h->t0));
-    HIP_TRY(hipEventCreate(&h->t1));
+    hipError_t e = hipSuccess;
+    for (int i = 0; i < kSlots && e == hipSuccess; ++i)
+        e = hipEventCreateWithFlags(&h->slots[i].done, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreate(&h->t0);
+    if (e == hipSuccess) e = hipEventCreate(&h->t1);
+    if (e != hipSuccess) {
+        rt_destroy(h);
+        return fail(RT_EHIP, "creating events failed: %s (%d)", hipGetErrorString(e), (int)e);
+    }
     *out = h;
     return RT_OK;
 }
@@ -516,6 +545,7 @@ int rt_grad_norm(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, float in
     rt_scalars one;
     memset(&one, 0, sizeof(one));
     one.inv_loss_scale = 1.0f;
+    uint64_t total_chunks = 0;
     for (uint32_t i = 0; i < n; ++i) {
         rt_tensor_desc& d = gd[i];
         if (d.g_dtype > RT_DT_F16) return fail(RT_EINVAL, "tensor %u: g_dtype %d unknown", i, d.g_dtype);
@@ -523,6 +553,8 @@ int rt_grad_norm(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, float in
         if (d.numel && ((uintptr_t)d.g % dtype_size(d.g_dtype)))
             return fail(RT_EINVAL, "tensor %u: g not aligned to its element size", i);
         if (d.numel / kChunkElems >= 0xFFFFFFFFull) return fail(RT_EUNSUPPORTED, "tensor %u: numel too large", i);
+        total_chunks += (d.numel + kChunkElems - 1) / kChunkElems;
+        if (total_chunks > kMaxGrid) return fail(RT_EUNSUPPORTED, "too many elements in one call");
         if (d.host_mask) return fail(RT_EINVAL, "tensor %u: host_mask set (grads must be device resident)", i);
         d.p = d.m = d.v = nullptr;
         d.noise_p = d.noise_m = d.noise_v = nullptr;
@@ -545,11 +577,9 @@ int rt_grad_norm(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, float in
     }
     int rc = dev_reserve(h->norm_partials, kNormPartials * sizeof(double));
     if (rc != RT_OK) return rc;
-    uint32_t grid = std::min<uint32_t>(kNormPartials, std::max<uint32_t>(plan.n_chunks, 1u));
-    if (plan.n_chunks == 0) {
-        HIP_TRY(hipMemsetAsync(h->norm_partials.ptr, 0, sizeof(double), stream));
-        grid = 1;
-    } else {
+    // With nothing to sum the finish kernel reads no partials (a total of zero).
+    const uint32_t grid = std::min<uint32_t>(kNormPartials, plan.n_chunks);
+    if (plan.n_chunks != 0) {
         TableSlot* slot = nullptr;
         rc = stage_image(h, plan, stream, &slot);
         if (rc != RT_OK) return rc;
@@ -709,15 +739,35 @@ static inline uint64_t tickets_done(const Streamed& st) {
     return st.ticket_word ? __atomic_load_n((const uint64_t*)st.ticket_word, __ATOMIC_ACQUIRE) : 0;
 }
 
+// Sleeps until ticket `want` has been published.  While the pipeline runs the host stays out
+// of the runtime: a thread spinning in a synchronise call, or polling events, was measured to
+// slow the copies down severalfold (the runtime resolves their cross-stream dependencies on
+// host threads).  The sleep is bounded: after kStallSeconds without a new ticket it returns
+// false and the caller falls back to a blocking synchronise, which also reports a failed device.
+static bool sleep_until_ticket(const Streamed& st, uint64_t want) {
+    constexpr double kStallSeconds = 60.0;
+    uint64_t seen = tickets_done(st);
+    auto last_progress = std::chrono::steady_clock::now();
+    while (seen < want) {
+        std::this_thread::sleep_for(std::chrono::microseconds(100));
+        const uint64_t now_done = tickets_done(st);
+        const auto now = std::chrono::steady_clock::now();
+        if (now_done != seen) {
+            seen = now_done;
+            last_progress = now;
+        } else if (std::chrono::duration<double>(now - last_progress).count() > kStallSeconds) {
+            return false;
+        }
+    }
+    return true;
+}
+
 static int streamed_wait(rt_handle* h) {
     Streamed& st = h->st;
     if (!st.ready) return RT_OK;
     HIP_TRY(hipSetDevice(h->device));
-    // Sleep until the last ticket has been published, then synchronise (which returns at
-    // once).  While the pipeline runs the host stays out of the runtime: a thread spinning
-    // in a synchronise call, or polling events, was measured to slow the copies down
-    // severalfold (the runtime resolves their cross-stream dependencies on host threads).
-    while (tickets_done(st) < st.tickets_issued) std::this_thread::sleep_for(std::chrono::microseconds(100));
+    (void)sleep_until_ticket(st, st.tickets_issued);
+    // returns at once when the last ticket is out; otherwise this is the blocking fallback
     HIP_TRY(hipStreamSynchronize(st.d2h));
     HIP_TRY(hipStreamSynchronize(st.comp));
     HIP_TRY(hipStreamSynchronize(st.h2d));
@@ -769,7 +819,8 @@ static int streamed_enqueue(rt_handle* h, const rt_tensor_desc* descs, uint32_t 
     for (int a = 0; a < 4; ++a)
         for (int b = 0; b < 2; ++b)
             if (stage_esize[a]) {
-                const size_t want = max_used * 4;  // sized for fp32 so dtype changes never realloc
+                // sized for fp32 (or wider) so that the common dtype changes never reallocate
+                const size_t want = max_used * std::max(4, stage_esize[a]);
                 if (want > st.stage[a][b].cap && st.pending) {
                     rc = streamed_wait(h);  // the buffer may be in use by an earlier asynchronous call
                     if (rc != RT_OK) return rc;
@@ -820,14 +871,19 @@ static int streamed_enqueue(rt_handle* h, const rt_tensor_desc* descs, uint32_t 
     size_t slot = st.ring.size();
     for (;;) {
         const uint64_t done_now = tickets_done(st);
+        uint64_t oldest = UINT64_MAX;
         for (size_t i = 0; i < st.ring.size(); ++i) {
             Streamed::TableRing& r = st.ring[i];
             if (r.in_flight && r.ticket <= done_now) r.in_flight = false;
+            if (r.in_flight) oldest = std::min(oldest, r.ticket);
             if (!r.in_flight && (slot == st.ring.size() || (st.ring[slot].host_cap < blob.size() && r.host_cap >= blob.size())))
                 slot = i;
         }
         if (slot != st.ring.size()) break;
-        std::this_thread::sleep_for(std::chrono::microseconds(100));
+        if (!sleep_until_ticket(st, oldest)) {
+            rc = streamed_wait(h);  // blocking fallback; frees every entry or reports the device error
+            if (rc != RT_OK) return rc;
+        }
     }
     Streamed::TableRing& tab = st.ring[slot];
     if (blob.size() > tab.host_cap) {

@@ -28,7 +28,7 @@ struct alignas(16) DevTensor {
     uint32_t tensor_id4;        // tensor_id * 4; + {0,1,2} selects p / m / v noise
     uint32_t set_idx;           // index into the DevScalars array
     uint32_t flags;
-    uint32_t pad;
+    uint32_t dtypes;            // p | g << 2 | m << 4 | v << 6 (RT_DT_*), read by the runtime-typed kernel
 };
 static_assert(sizeof(DevTensor) == 128, "DevTensor layout");
 

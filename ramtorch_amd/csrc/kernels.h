@@ -412,6 +412,113 @@ __global__ __launch_bounds__(kThreads) void sr_adamw_generic_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// Runtime-typed kernel: tensors whose param or states are kept in fp16 or fp64.
+// The reference upcasts every dtype to fp32 (adamw.py:160-170) and writes
+// anything that is not bf16 back with a plain copy_ (adamw.py:208,214,221-222):
+// fp16 is rounded to nearest even (v_cvt_f16_f32), fp64 widened exactly; an
+// fp64 input is rounded to nearest even on the way in.  Such layouts are rare,
+// so this is one kernel with a per-tensor dtype switch instead of another 200
+// instantiations: a lane owns one Philox block of 8 elements, as in the
+// kernels above, and moves them element by element.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float load_any(uint64_t base, uint32_t dt, uint64_t idx) {
+    switch (dt) {
+        case RT_DT_BF16: return u2f(ldg16(base + idx * 2) << 16);
+        case RT_DT_F16: return (float)__builtin_bit_cast(_Float16, (uint16_t)ldg16(base + idx * 2));
+        case RT_DT_F64: return (float)*(const RT_GLOBAL double*)(base + idx * 8);
+        default: return ldg32f(base + idx * 4);
+    }
+}
+
+__device__ __forceinline__ void store_any(uint64_t base, uint32_t dt, uint64_t idx, float x, uint32_t noise16) {
+    switch (dt) {
+        case RT_DT_BF16: stg16(base + idx * 2, (f2u(x) + noise16) >> 16); break;
+        case RT_DT_F16: stg16(base + idx * 2, __builtin_bit_cast(uint16_t, (_Float16)x)); break;
+        case RT_DT_F64: *(RT_GLOBAL double*)(base + idx * 8) = (double)x; break;
+        default: stg32f(base + idx * 4, x); break;
+    }
+}
+
+__device__ __forceinline__ uint32_t noise_field(const u32x4& z, int j) {
+    const uint32_t w = (j >> 1) == 0 ? z.x : (j >> 1) == 1 ? z.y : (j >> 1) == 2 ? z.z : z.w;
+    return (j & 1) ? (w >> 16) : (w & 0xFFFFu);
+}
+
+template <int NOISE>
+__global__ __launch_bounds__(kThreads) void sr_adamw_any_kernel(
+    const DevTensor* __restrict__ tensors, const ChunkRef* __restrict__ chunks,
+    const DevScalars* __restrict__ sets, uint32_t seed_lo, uint32_t seed_hi,
+    const float* __restrict__ clip_coef, const uint32_t* __restrict__ skip) {
+    if (skip != nullptr && *skip != 0u) return;
+    const ChunkRef cr = chunks[blockIdx.x];
+    const DevTensor& t = tensors[cr.tensor];
+    const DevScalars& set = sets[t.set_idx];
+    const rt_scalars s = set.s;
+    const bool do_clip = clip_coef != nullptr;
+    const float coef = do_clip ? *clip_coef : 1.0f;
+    const bool do_unscale = s.inv_loss_scale != 1.0f;
+    const uint32_t pdt = t.dtypes & 3u, gdt = (t.dtypes >> 2) & 3u, mdt = (t.dtypes >> 4) & 3u,
+                   vdt = (t.dtypes >> 6) & 3u;
+    const uint64_t n = t.numel;
+    const uint64_t chunk_base = (uint64_t)cr.chunk * kChunkElems;
+#pragma unroll 1
+    for (int it = 0; it < kItersPerChunk; ++it) {
+        const uint64_t i = chunk_base + (uint64_t)(it * kThreads + (int)threadIdx.x) * kVec;
+        if (i >= n) break;
+        u32x4 zp = 0, zm = 0, zv = 0;
+        if constexpr (NOISE == RT_NOISE_PHILOX) {
+            const uint64_t blk = t.block_base + (i >> 3);
+            const uint32_t b0 = (uint32_t)blk, b1 = (uint32_t)(blk >> 32);
+            if (pdt == RT_DT_BF16) zp = philox4x32_10(b0, b1, t.tensor_id4 + 0u, set.step, seed_lo, seed_hi);
+            if (mdt == RT_DT_BF16) zm = philox4x32_10(b0, b1, t.tensor_id4 + 1u, set.step, seed_lo, seed_hi);
+            if (vdt == RT_DT_BF16) zv = philox4x32_10(b0, b1, t.tensor_id4 + 2u, set.step, seed_lo, seed_hi);
+        }
+        uint64_t row = 0, rem = 0;
+        if (t.row_mean != 0) {
+            const uint64_t e0 = (t.block_base << 3) + i;
+            row = e0 / t.row_len;
+            rem = e0 - row * t.row_len;
+        }
+#pragma unroll 1
+        for (int j = 0; j < kVec; ++j) {
+            const uint64_t e = i + j;
+            if (e >= n) break;
+            float p = load_any(t.p, pdt, e);
+            float g = load_any(t.g, gdt, e);
+            float m = load_any(t.m, mdt, e);
+            float v = load_any(t.v, vdt, e);
+            if (do_unscale) g = g * s.inv_loss_scale;
+            if (do_clip) g = g * coef;
+            if (t.row_mean != 0) {
+                const float mc = ldg32f(t.row_mean + row * 4) * s.centralization;
+                g = g - mc;
+                if (++rem == t.row_len) {
+                    rem = 0;
+                    ++row;
+                }
+            }
+            update1(p, g, m, v, s);
+            if (t.dp != 0) stg32f(t.dp + e * 4, p);
+            if (t.dm != 0) stg32f(t.dm + e * 4, m);
+            if (t.dv != 0) stg32f(t.dv + e * 4, v);
+            uint32_t np16, nm16, nv16;
+            if constexpr (NOISE == RT_NOISE_EXPLICIT) {
+                np16 = pdt == RT_DT_BF16 ? ldg16(t.np + e * 2) : 0u;
+                nm16 = mdt == RT_DT_BF16 ? ldg16(t.nm + e * 2) : 0u;
+                nv16 = vdt == RT_DT_BF16 ? ldg16(t.nv + e * 2) : 0u;
+            } else {
+                np16 = noise_field(zp, j);
+                nm16 = noise_field(zm, j);
+                nv16 = noise_field(zv, j);
+            }
+            store_any(t.p, pdt, e, p, np16);
+            store_any(t.m, mdt, e, m, nm16);
+            store_any(t.v, vdt, e, v, nv16);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Copies a table image from pinned host memory (read over the host link by the
 // kernel itself) into device memory.  The streamed pipeline uses this instead
 // of a DMA copy: a small hipMemcpyAsync queued between the large H2D / D2H

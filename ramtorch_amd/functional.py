@@ -15,6 +15,9 @@ import torch
 from . import _native as N
 
 _DT_CODE = {torch.bfloat16: N.RT_DT_BF16, torch.float32: N.RT_DT_F32, torch.float16: N.RT_DT_F16}
+#: params and states may also be fp64 (upcast / plain copy_ semantics of adamw.py:160-170, 208-222)
+_DT_CODE_PMV = dict(_DT_CODE)
+_DT_CODE_PMV[torch.float64] = N.RT_DT_F64
 
 #: numpy mirror of ``rt_tensor_desc`` (same field order and offsets)
 DESC_DTYPE = np.dtype(
@@ -30,10 +33,10 @@ assert DESC_DTYPE.itemsize == ctypes.sizeof(N.RtTensorDesc)
 
 def dtype_code(dt: torch.dtype, what: str) -> int:
     try:
-        return _DT_CODE[dt]
+        return (_DT_CODE if what == "grad" else _DT_CODE_PMV)[dt]
     except KeyError:
-        raise NotImplementedError(f"{what} dtype {dt} is not supported by the HIP step "
-                                  "(bf16 / fp32; fp16 for gradients only)") from None
+        raise NotImplementedError(f"{what} dtype {dt} is not supported by the HIP step (bf16 / fp32 / fp16; "
+                                  "fp64 for params and states)") from None
 
 
 def make_scalars(lr: float, betas: Tuple[float, float], eps: float, weight_decay: float, step: int,
@@ -104,8 +107,6 @@ def pack_descs(entries: Sequence[Entry], streamed: bool) -> np.ndarray:
     for i, e in enumerate(entries):
         if e.g.numel() != e.p.numel() or e.m.numel() != e.p.numel() or e.v.numel() != e.p.numel():
             raise ValueError(f"tensor {i}: p/g/m/v element counts differ")
-        if torch.float16 in (e.p.dtype, e.m.dtype, e.v.dtype):
-            raise NotImplementedError("fp16 params/states are not supported by the HIP step (bf16 or fp32)")
         if e.noise is not None:
             for name, t, tgt in zip(("noise_p", "noise_m", "noise_v"), e.noise, (e.p, e.m, e.v)):
                 if t is None:

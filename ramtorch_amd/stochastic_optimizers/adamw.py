@@ -203,7 +203,7 @@ class AdamW(Optimizer):
         r.p, r.state, r.m, r.v, r.tensor_id = p, state, m, v, tensor_id
         r.p_ptr, r.m_ptr, r.v_ptr, r.numel = p.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel()
         r.dev = _compute_device_index(p)
-        ok_dt = (torch.bfloat16, torch.float32)
+        ok_dt = F._DT_CODE_PMV
         r.plain = (p.is_cuda and m.is_cuda and v.is_cuda and m.device == p.device and v.device == p.device
                    and p.is_contiguous() and m.is_contiguous() and v.is_contiguous()
                    and p.dtype in ok_dt and m.dtype in ok_dt and v.dtype in ok_dt

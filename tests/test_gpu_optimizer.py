@@ -73,6 +73,58 @@ def test_three_steps_match_the_reference_op_sequence():
             assert opt.state[p]["step"] == step
 
 
+def _nmis_any(a, b):
+    a, b = a.detach().cpu().contiguous(), b.detach().cpu().contiguous()
+    assert a.shape == b.shape and a.dtype == b.dtype, (a.shape, b.shape, a.dtype, b.dtype)
+    it = {2: torch.int16, 4: torch.int32, 8: torch.int64}[a.element_size()]
+    return int((a.view(it) != b.view(it)).sum())
+
+
+@pytest.mark.parametrize("p_dt,s_dt", [(torch.float16, torch.float16), (torch.float32, torch.float16),
+                                        (torch.float64, torch.float64), (torch.bfloat16, torch.float16),
+                                        (torch.float16, torch.bfloat16)])
+@pytest.mark.parametrize("where", ["cuda", "cpu"])
+def test_other_param_and_state_dtypes_match_the_reference_op_sequence(p_dt, s_dt, where):
+    """The reference accepts any float dtype: everything is upcast to fp32 (adamw.py:160-170) and what
+    is not bf16 is written back with a plain copy_ (adamw.py:208,214,221-222).  Two steps, GPU
+    states and host-resident (pinned) states, against the same ATen calls on the GPU."""
+    shapes = [(40, 33), (8192 + 11,), (5,)]
+    ps, grads, ref_p = [], [], []
+    for i, shp in enumerate(shapes):
+        n = int(np.prod(shp))
+        p, g, _, _ = oracle.synth_inputs(n, 700 + i)
+        p32 = torch.from_numpy(oracle.bf16_to_f32(p).copy()).view(shp) * 1.001
+        t = p32.to(p_dt)
+        if where == "cpu":
+            t = t.pin_memory()
+        else:
+            t = t.cuda()
+        ps.append(torch.nn.Parameter(t, requires_grad=False))
+        ref_p.append(t.detach().clone().cuda())
+        grads.append(dev16(g).view(shp))
+    opt = ramtorch_amd.AdamW(ps, lr=1e-3, dtype=s_dt, storage_device=where, stream_chunk_bytes=16384)
+    ref_m = [torch.zeros_like(p, dtype=s_dt) for p in ref_p]
+    ref_v = [torch.zeros_like(p, dtype=s_dt) for p in ref_p]
+    for step in (1, 2):
+        noise, gmap = {}, {}
+        for i, p in enumerate(ps):
+            gmap[p] = (grads[i].float() * (1.0 + 0.25 * step)).bfloat16()
+            noise[p] = tuple(torch.randint(-32768, 32768, p.shape, dtype=torch.int16, device="cuda",
+                                           generator=torch.Generator("cuda").manual_seed(step * 10 + i * 3 + k))
+                             for k in range(3))
+        opt.step(noise=noise, grads=gmap)
+        torch.cuda.synchronize()
+        for i, p in enumerate(ps):
+            st = opt.state[p]
+            assert st["ema"].dtype == s_dt and st["ema_squared"].dtype == s_dt and p.dtype == p_dt
+            assert st["ema"].device.type == where
+            torch_ops.reference_step_ops(ref_p[i], gmap[p], ref_m[i], ref_v[i], lr=1e-3, betas=(0.9, 0.999),
+                                         eps=1e-8, weight_decay=1e-2, step=step, noise=noise[p])
+            assert _nmis_any(p.detach(), ref_p[i]) == 0, f"step {step} param {i}"
+            assert _nmis_any(st["ema"], ref_m[i]) == 0, f"step {step} ema {i}"
+            assert _nmis_any(st["ema_squared"], ref_v[i]) == 0, f"step {step} ema_squared {i}"
+
+
 def test_skipped_and_sparse_gradients():
     ps, grads = _make_params([(32, 8), (40,)], 200)
     opt = ramtorch_amd.AdamW(ps, storage_device="cuda")

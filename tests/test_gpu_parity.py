@@ -55,7 +55,7 @@ def run_both(handle, p, g, m, v, *, hp=HP0, step=10, noise=None, seed=1234, tens
     tdt = {oracle.DT_BF16: torch.bfloat16, oracle.DT_F16: torch.float16}
 
     def up(a, code):
-        return torch.from_numpy(a.copy()).cuda() if code == oracle.DT_F32 else dev16(a, tdt[code])
+        return torch.from_numpy(a.copy()).cuda() if code in (oracle.DT_F32, oracle.DT_F64) else dev16(a, tdt[code])
 
     P, G, M, V = up(p, p_dtype), up(g, g_dtype), up(m, m_dtype), up(v, v_dtype)
     n = p.size
@@ -72,8 +72,13 @@ def run_both(handle, p, g, m, v, *, hp=HP0, step=10, noise=None, seed=1234, tens
     d = oracle.step_tensor(po, g, mo, vo, sco, p_dtype=p_dtype, g_dtype=g_dtype, m_dtype=m_dtype, v_dtype=v_dtype,
                            clip_coef=1.0 if clip_coef is None else clip_coef, noise=noise, seed=seed, step=step,
                            tensor_id=tensor_id, debug=True)
-    got = [bits32(t) if t.dtype == torch.float32 else bits16(t) for t in (P, M, V)]
-    want = [a.view(np.uint32) if a.dtype == np.float32 else a for a in (po, mo, vo)]
+    def tbits(t):
+        if t.dtype == torch.float64:
+            return t.detach().cpu().contiguous().numpy().view(np.uint64)
+        return bits32(t) if t.dtype == torch.float32 else bits16(t)
+    nbits = {np.dtype(np.float32): np.uint32, np.dtype(np.float64): np.uint64, np.dtype(np.uint16): np.uint16}
+    got = [tbits(t) for t in (P, M, V)]
+    want = [a.view(nbits[a.dtype]) for a in (po, mo, vo)]
     return got, want, (None if dbg is None else [bits32(t) for t in dbg]), [x.view(np.uint32) for x in d]
 
 
@@ -207,6 +212,12 @@ def test_hyperparameters(handle, hp, step):
     (oracle.DT_BF16, oracle.DT_F16, oracle.DT_BF16, oracle.DT_BF16),
     (oracle.DT_F32, oracle.DT_BF16, oracle.DT_BF16, oracle.DT_BF16),
     (oracle.DT_BF16, oracle.DT_BF16, oracle.DT_F32, oracle.DT_BF16),
+    # fp16 / fp64 params and states: upcast like everything else, plain copy_ on the way back
+    # (adamw.py:208,214,221-222) -- the runtime-typed kernel
+    (oracle.DT_F16, oracle.DT_F16, oracle.DT_F16, oracle.DT_F16),
+    (oracle.DT_BF16, oracle.DT_BF16, oracle.DT_F16, oracle.DT_F16),
+    (oracle.DT_F64, oracle.DT_F32, oracle.DT_BF16, oracle.DT_F64),
+    (oracle.DT_F16, oracle.DT_BF16, oracle.DT_F64, oracle.DT_F32),
 ])
 @pytest.mark.parametrize("mode", ["explicit", "philox"])
 def test_dtype_combinations(handle, p_dt, g_dt, m_dt, v_dt, mode):
@@ -218,6 +229,8 @@ def test_dtype_combinations(handle, p_dt, g_dt, m_dt, v_dt, mode):
             return (oracle.bf16_to_f32(a) * np.float32(1.0009765625)).astype(np.float32)  # not bf16-exact
         if dt == oracle.DT_F16:
             return oracle.bf16_to_f32(a).astype(np.float16).view(np.uint16)
+        if dt == oracle.DT_F64:  # not representable in fp32: the upcast to fp32 has to round
+            return oracle.bf16_to_f32(a).astype(np.float64) * (1.0 + 2.0 ** -30)
         return a
     p, g, m, v = conv(p, p_dt), conv(g, g_dt), conv(m, m_dt), conv(v, v_dt)
     noise = oracle.synth_noise(n, 31) if mode == "explicit" else None
@@ -225,6 +238,30 @@ def test_dtype_combinations(handle, p_dt, g_dt, m_dt, v_dt, mode):
         got, want, dbg, pre = run_both(handle, p, g, m, v, noise=noise, p_dtype=p_dt, g_dtype=g_dt, m_dtype=m_dt,
                                        v_dtype=v_dt, debug=debug)
         assert_same(got, want, dbg, pre, f"dtypes {p_dt}{g_dt}{m_dt}{v_dt} {mode}")
+
+
+def test_fp16_param_overflow_and_gradual_underflow(handle):
+    """An fp16 param written back past the fp16 range becomes inf, tiny values land on
+    fp16 subnormals (round to nearest even), as Tensor.copy_ does."""
+    n = 4096 + 5
+    p, g, m, v = oracle.synth_inputs(n, 77)
+    p16 = oracle.bf16_to_f32(p).astype(np.float16)
+    p16[:8] = [65504.0, -65504.0, 6e-8, -6e-8, 6.1e-5, 1.2e-7, 0.0, -0.0]
+    g16 = oracle.bf16_to_f32(g).astype(np.float16)
+    g16[:2] = [-60000.0, 60000.0]  # pushes the two largest values over the edge
+    g16[8:12] = [6e-8, 1e-6, -3e-7, 2e-5]  # ema = 0.1 * g: fp16 subnormals and zero
+    hp = dict(lr=100.0, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0)
+    m0 = np.zeros(n, np.uint16)
+    got, want, dbg, pre = run_both(handle, p16.view(np.uint16), g16.view(np.uint16), m0, m0.copy(), hp=hp, step=1,
+                                   p_dtype=oracle.DT_F16, g_dtype=oracle.DT_F16, m_dtype=oracle.DT_F16,
+                                   v_dtype=oracle.DT_F16)
+    assert_same(got, want, dbg, pre, "fp16 edges")
+    out = got[0].view(np.float16)
+    assert np.isinf(out[0]) and out[0] > 0 and np.isinf(out[1]) and out[1] < 0
+    assert np.isinf(got[2].view(np.float16)[0])  # g*g overflows fp16 in ema_squared as well
+    ema = got[1].view(np.float16)[8:12]
+    # below half the smallest subnormal -> 0; a subnormal; exactly -2^-25, a tie -> -0 (even)
+    assert ema[0] == 0 and 0 < ema[1] < 6.1e-5 and got[1][10] == 0x8000
 
 
 def test_loss_scale_and_clip_coefficient(handle):

@@ -210,8 +210,13 @@ def test_pack_descs_rejects_bad_inputs():
     assert d["host_mask"][0] == 15 and d["numel"][0] == 8 and d["p"][0] == e.p.data_ptr()
     with pytest.raises(ValueError, match="element counts"):
         F.pack_descs([F.Entry(p=t(8), g=t(9), m=t(8), v=t(8), step=1, scalars_idx=0, tensor_id=0)], streamed=True)
+    # fp16 / fp64 params and states are valid (plain copy_ on write-back, adamw.py:208-222) ...
+    d = F.pack_descs([F.Entry(p=t(8, torch.float16), g=t(8), m=t(8, torch.float64), v=t(8, torch.float32), step=1,
+                              scalars_idx=0, tensor_id=0)], streamed=True)
+    assert (d["p_dtype"][0], d["g_dtype"][0], d["m_dtype"][0], d["v_dtype"][0]) == (2, 0, 3, 1)
+    # ... other dtypes are not, and neither is an fp64 gradient at this level (AdamW.step downcasts it first)
     with pytest.raises(NotImplementedError):
-        F.pack_descs([F.Entry(p=t(8, torch.float16), g=t(8), m=t(8), v=t(8), step=1, scalars_idx=0, tensor_id=0)],
+        F.pack_descs([F.Entry(p=t(8, torch.int16), g=t(8), m=t(8), v=t(8), step=1, scalars_idx=0, tensor_id=0)],
                      streamed=True)
     with pytest.raises(NotImplementedError):
         F.pack_descs([F.Entry(p=t(8), g=t(8, torch.float64), m=t(8), v=t(8), step=1, scalars_idx=0, tensor_id=0)],

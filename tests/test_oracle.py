@@ -309,6 +309,78 @@ def test_f16_gradient_decode():
     np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+def test_f32_to_f16_matches_numpy_and_torch():
+    """fp16 params / states take a plain copy_ (adamw.py:208,214,221-222): round to nearest even
+    with gradual underflow.  Pinned against numpy's and torch's own conversions on every
+    high-half pattern crossed with the low halves that decide the rounding, plus random bits."""
+    hi = np.arange(1 << 16, dtype=np.uint32) << 16
+    lows = np.array([0x0000, 0x0001, 0x0FFF, 0x1000, 0x1001, 0x1FFF, 0x2000, 0x2FFF, 0x3000, 0x3001, 0x7FFF,
+                     0x8000, 0x8001, 0xEFFF, 0xF000, 0xF001, 0xFFFF], np.uint32)
+    bits = (hi[:, None] | lows[None, :]).ravel()
+    rng = np.random.default_rng(3)
+    bits = np.concatenate([bits, rng.integers(0, 1 << 32, 2_000_000, dtype=np.uint64).astype(np.uint32)])
+    x = bits.view(np.float32)
+    finite = ~np.isnan(x)  # NaN payloads are not part of the contract
+    got = oracle.f32_to_f16_rne(x)
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    np.testing.assert_array_equal(got[finite], want[finite])
+    want_t = torch.from_numpy(x.copy()).to(torch.float16).view(torch.int16).numpy().view(np.uint16)
+    np.testing.assert_array_equal(got[finite], want_t[finite])
+    nan16 = got[~finite]
+    assert np.all((nan16 & 0x7C00) == 0x7C00) and np.all((nan16 & 0x03FF) != 0)
+
+
+@pytest.mark.parametrize("dts", [("f16", "f16", "f16"), ("f64", "f16", "f32"), ("bf16", "f64", "f16"),
+                                 ("f16", "bf16", "f64")])
+def test_fp16_and_fp64_targets_take_a_plain_copy(dts):
+    """Write-back dtype only changes the last conversion: the fp32 result (debug output) is the
+    same as in the all-fp32 run fed the same upcast inputs, and the stored value is its plain
+    conversion (numpy's), not a stochastic rounding."""
+    n = 4099
+    pb, gb, mb, vb = oracle.synth_inputs(n, 21)
+    f32 = [oracle.bf16_to_f32(a).copy() for a in (pb, gb, mb, vb)]
+    f32[0][:4] = [70000.0, -70000.0, 1e-7, -3e-8]  # fp16 overflow and gradual underflow of the param
+    code = {"bf16": oracle.DT_BF16, "f32": oracle.DT_F32, "f16": oracle.DT_F16, "f64": oracle.DT_F64}
+
+    def store(x32, dt):
+        if dt == "f16":
+            with np.errstate(over="ignore"):
+                return x32.astype(np.float16).view(np.uint16).copy()
+        if dt == "f64":
+            return x32.astype(np.float64)
+        if dt == "bf16":
+            return oracle.f32_to_bf16_rne(x32)
+        return x32.copy()
+
+    def load(a, dt):
+        if dt == "f16":
+            return a.view(np.float16).astype(np.float32)
+        if dt == "f64":
+            return a.astype(np.float32)
+        if dt == "bf16":
+            return oracle.bf16_to_f32(a)
+        return a
+
+    arrs = [store(f32[0], dts[0]), store(f32[2], dts[1]), store(f32[3], dts[2])]
+    ups = [load(a, dt).copy() for a, dt in zip(arrs, dts)]
+    sc = oracle.scalars_from_hparams(step=7, **HP0)
+    ref = oracle.step_tensor(ups[0], f32[1], ups[1], ups[2], sc, p_dtype=oracle.DT_F32, g_dtype=oracle.DT_F32,
+                             m_dtype=oracle.DT_F32, v_dtype=oracle.DT_F32, seed=5, step=7, debug=True)
+    dbg = oracle.step_tensor(arrs[0], f32[1], arrs[1], arrs[2], sc, p_dtype=code[dts[0]], g_dtype=oracle.DT_F32,
+                             m_dtype=code[dts[1]], v_dtype=code[dts[2]], seed=5, step=7, tensor_id=3, debug=True)
+    for k in range(3):
+        np.testing.assert_array_equal(dbg[k].view(np.uint32), ref[k].view(np.uint32))
+        if dts[k] == "bf16":
+            nz = oracle.philox_noise_array(5, 7, 3, k, 0, n)
+            want = ((dbg[k].view(np.uint32).astype(np.uint64) + nz) >> 16).astype(np.uint16)
+            np.testing.assert_array_equal(arrs[k], want)
+        else:
+            w = store(dbg[k], dts[k])
+            np.testing.assert_array_equal(arrs[k].view(np.uint16 if dts[k] == "f16" else arrs[k].dtype),
+                                          w.view(np.uint16 if dts[k] == "f16" else w.dtype))
+
+
 def test_grad_sumsq_and_clip_coef():
     g = oracle.f32_to_bf16_rne(np.random.default_rng(0).normal(0, 1e-3, 10_000).astype(np.float32) * 1024)
     want = float(np.sum((oracle.bf16_to_f32(g).astype(np.float64) / 1024) ** 2))
