@@ -4,7 +4,8 @@
 
 hipcc cross-compiles for gfx950 without a GPU.  The library lands next to the
 sources as ``ramtorch_amd/_lib/libramtorch_sr_adamw.so`` and is loaded with
-ctypes (see ``_native.py``); nothing is installed outside the tree.
+ctypes (see ``_native.py``); nothing is installed outside the tree.  A second,
+optional artefact is a small CPython extension built with g++ (``build_gather``).
 """
 from __future__ import annotations
 
@@ -59,6 +60,40 @@ def build(verbose: bool = False, extra_flags=()) -> str:
     return LIB_PATH
 
 
+# ---- optional CPython helper (plain g++; links against the installed torch) -------------------
+GATHER_SRC = os.path.join(CSRC, "host_gather.cpp")
+
+
+def gather_path() -> str:
+    import sysconfig
+    return os.path.join(LIB_DIR, "_rt_gather" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_gather(verbose: bool = False) -> str:
+    """Compiles csrc/host_gather.cpp, the descriptor gatherer AdamW.step uses for
+    parameter sets with many tensors.  It reads tensors through torch's C++ API, so it
+    is tied to the installed torch build."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension
+
+    os.makedirs(LIB_DIR, exist_ok=True)
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-function",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           "-I" + sysconfig.get_paths()["include"]]
+    cmd += ["-I" + i for i in cpp_extension.include_paths()]
+    cmd += [GATHER_SRC, "-o", gather_path(), "-L" + torch_lib, "-ltorch_python", "-ltorch", "-ltorch_cpu", "-lc10",
+            "-Wl,-rpath," + torch_lib]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"building the gather helper failed ({res.returncode}):\n{res.stdout}\n{res.stderr}")
+    return gather_path()
+
+
 def is_stale() -> bool:
     if not os.path.exists(LIB_PATH):
         return True
@@ -69,3 +104,4 @@ def is_stale() -> bool:
 
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_gather(verbose=True))

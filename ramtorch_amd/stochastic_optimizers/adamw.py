@@ -16,6 +16,7 @@ import numpy as np
 import torch
 from torch.optim import Optimizer
 
+from .. import _gather as G
 from .. import _native as N
 from .. import functional as F
 
@@ -115,6 +116,10 @@ class AdamW(Optimizer):
         self.max_inflight_bytes = 2 << 30  # gradients kept alive for updates still in flight (step_param)
         self.max_inflight_calls = 2       # staging chunks handed to the copy pipeline and not finished yet
         self._poll_seconds = 0.0002       # completion is read from host memory; no runtime call while waiting
+        self.gather_min_tensors = 256     # from this many parameters on, step() gathers descriptors in C++
+        self._gather_bufs = {}            # device -> descriptor rows the gatherer fills
+        self._gather_stat = None
+        self._state_lists = {}
         self._stepped_early = set()       # id(param) updated by step_param since the last step()
         self._inflight = []               # (device, ticket, bytes, tensors kept alive)
         self._early_batch = {}            # device -> [[entry, scalars, handed-over elements], ...], pending elements
@@ -129,6 +134,10 @@ class AdamW(Optimizer):
         super().__setstate__(state)
         self._recs = None
         self._desc_cache = {}
+        self._state_lists = {}
+        self.__dict__.setdefault("gather_min_tensors", 256)
+        self.__dict__.setdefault("_gather_bufs", {})
+        self.__dict__.setdefault("_gather_stat", None)
 
     def state_dict(self):
         """Same layout as the reference (``state`` with ``step / ema / ema_squared`` per
@@ -165,6 +174,7 @@ class AdamW(Optimizer):
                     st[k] = t
         self._recs = None
         self._desc_cache = {}
+        self._state_lists = {}
 
     # -- state ---------------------------------------------------------------------
     def _new_state_tensor(self, p: torch.Tensor) -> torch.Tensor:
@@ -230,6 +240,7 @@ class AdamW(Optimizer):
             recs.append(row)
         self._recs = recs
         self._desc_cache = {}
+        self._state_lists = {}
         return recs
 
     # -- step ----------------------------------------------------------------------
@@ -268,13 +279,40 @@ class AdamW(Optimizer):
         extras = noise is not None or debug_out is not None
         dt_code = F._DT_CODE
 
+        # Large groups of plain GPU tensors are walked in C++ when the helper is built; it writes
+        # their descriptor rows and advances their step counts, and leaves the rest to the loop below.
+        gather = None
+        if (grads is None and not extras and not early and self.max_grad_norm is None
+                and sum(len(g["params"]) for g in self.param_groups) >= self.gather_min_tensors):
+            gather = G.module()
+        gathered: Dict[int, list] = {}    # dev -> [descriptor buffer, rows used]
+
         with torch.no_grad():
             for gi, group in enumerate(self.param_groups):
                 beta1, beta2 = group["betas"]
                 lr, eps, wd, cen = group["lr"], group["eps"], group["weight_decay"], group["centralization"]
                 row = recs[gi]
                 last_step, last_si = None, -1
-                for k, p in enumerate(group["params"]):
+                plist = group["params"]
+                work = enumerate(plist)
+                if gather is not None and cen == 0 and row and row[0].plain and isinstance(plist, list):
+                    dev = row[0].dev
+                    slot = gathered.get(dev)
+                    if slot is None:
+                        slot = gathered[dev] = [self._gather_buffer(dev), 0]
+                    buf, used = slot
+                    status = self._gather_status(len(plist))
+                    n_rows, new_steps = gather.gather_group(
+                        plist, self._state_list(gi), dev, buf.ctypes.data + used * buf.itemsize, len(buf) - used,
+                        status.ctypes.data, len(scalars), row[0].tensor_id)
+                    slot[1] = used + n_rows
+                    for st in new_steps:
+                        scalar_key[(gi, st, lr, beta1, beta2, eps, wd, cen)] = len(scalars)
+                        scalars.append(F.make_scalars(lr, (beta1, beta2), eps, wd, st, centralization=cen,
+                                                      inv_loss_scale=inv_loss_scale))
+                    rest = np.flatnonzero(status[:len(plist)] == gather.PYTHON)
+                    work = ((int(k), plist[int(k)]) for k in rest)
+                for k, p in work:
                     grad = grads.get(p, p.grad) if grads is not None else p.grad
                     if grad is None:
                         continue  # adamw.py:114: skipped, and its step count does not advance
@@ -353,12 +391,15 @@ class AdamW(Optimizer):
                     (resident if on_gpu else streamed).setdefault(dev, []).append(e)
 
             explicit = noise is not None
-            for dev in sorted(set(plain) | set(resident) | set(streamed)):
+            for dev in sorted(set(plain) | set(resident) | set(streamed) | set(gathered)):
                 h = _handle(dev)
                 with torch.cuda.device(dev):
                     res, stm = resident.get(dev, []), streamed.get(dev, [])
                     lane = plain.get(dev)
                     descs = self._plain_descs(dev, lane) if lane is not None else None
+                    if dev in gathered and gathered[dev][1]:
+                        d0 = gathered[dev][0][:gathered[dev][1]]
+                        descs = d0 if descs is None else np.concatenate([d0, descs])
                     if res:
                         d2 = F.pack_descs(res, streamed=False)
                         descs = d2 if descs is None else np.concatenate([descs, d2])
@@ -530,6 +571,27 @@ class AdamW(Optimizer):
             with torch.cuda.device(dev):
                 _handle(dev).streamed_wait()
         self._inflight = []
+
+    def _gather_buffer(self, dev: int) -> np.ndarray:
+        """Descriptor rows the C++ gatherer fills for one device (one row per parameter at most)."""
+        n = sum(len(g["params"]) for g in self.param_groups)
+        buf = self._gather_bufs.get(dev)
+        if buf is None or len(buf) < n:
+            buf = self._gather_bufs[dev] = np.zeros(n, F.DESC_DTYPE)
+        return buf
+
+    def _gather_status(self, n: int) -> np.ndarray:
+        st = self._gather_stat
+        if st is None or len(st) < n:
+            st = self._gather_stat = np.zeros(n, np.uint8)
+        return st
+
+    def _state_list(self, gi: int) -> list:
+        """The state dicts of group ``gi`` in parameter order (cached with the records)."""
+        lst = self._state_lists.get(gi)
+        if lst is None or len(lst) != len(self._recs[gi]):
+            lst = self._state_lists[gi] = [r.state for r in self._recs[gi]]
+        return lst
 
     def _plain_descs(self, dev: int, lane) -> np.ndarray:
         """Descriptor array of the plain lane.  The columns that describe p / m / v are

@@ -341,3 +341,52 @@ def test_copy_stochastic():
     cpu_tgt = torch.empty(n, dtype=torch.bfloat16)
     ramtorch_amd.copy_stochastic_(cpu_tgt, src, seed=42)
     assert nmis(cpu_tgt, tgt.cpu()) == 0
+
+
+def test_gathered_step_equals_the_python_loop():
+    """With many tensors AdamW.step collects descriptors in C++.  Same parameters through that
+    path and through the Python loop (gatherer switched off): identical bits and step counts,
+    also with skipped gradients, a non-contiguous parameter, two groups."""
+    from ramtorch_amd import _gather as G
+    if G.module() is None:
+        pytest.skip("gather helper not built")
+    rng = np.random.default_rng(11)
+    lens = [int(x) for x in np.exp(rng.uniform(0, np.log(20000), 600)).astype(np.int64).clip(1, 20000)]
+
+    def make():
+        ps = []
+        for i, n in enumerate(lens):
+            p, g, _, _ = oracle.synth_inputs(n, 5000 + i)
+            t = dev16(p)
+            if i == 17:
+                t = torch.stack([t, t], 1)[:, 0]  # not contiguous
+            q = torch.nn.Parameter(t, requires_grad=False)
+            ps.append(q)
+        return ps
+
+    def set_grads(ps, step):
+        for i, (p, n) in enumerate(zip(ps, lens)):
+            if (i + step) % 11 == 0:
+                p.grad = None
+                continue
+            _, g, _, _ = oracle.synth_inputs(n, 5000 + i + 100 * step)
+            p.grad = dev16(g).view(p.shape)
+
+    a, b = make(), make()
+    kw = dict(storage_device="cuda", seed=77)
+    oa = ramtorch_amd.AdamW([{"params": a[:400]}, {"params": a[400:], "lr": 3e-4, "weight_decay": 0.0}], **kw)
+    ob = ramtorch_amd.AdamW([{"params": b[:400]}, {"params": b[400:], "lr": 3e-4, "weight_decay": 0.0}], **kw)
+    ob.gather_min_tensors = 10 ** 9  # Python loop only
+    assert oa.gather_min_tensors <= len(a)
+    for step in (1, 2, 3):
+        set_grads(a, step)
+        set_grads(b, step)
+        oa.step()
+        ob.step()
+        torch.cuda.synchronize()
+        for i, (p, q) in enumerate(zip(a, b)):
+            assert oa.state[p]["step"] == ob.state[q]["step"], (step, i)
+            assert nmis(p.detach(), q.detach()) == 0, (step, i)
+            assert nmis(oa.state[p]["ema"], ob.state[q]["ema"]) == 0, (step, i)
+            assert nmis(oa.state[p]["ema_squared"], ob.state[q]["ema_squared"]) == 0, (step, i)
+    assert max(oa.state[p]["step"] for p in a) == 3 and min(oa.state[p]["step"] for p in a) >= 2

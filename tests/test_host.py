@@ -267,3 +267,63 @@ def test_streamed_plan_rejects_bad_chunk_size():
     d = np.zeros(1, F.DESC_DTYPE)
     with pytest.raises(N.NativeError):
         N.streamed_plan(d.ctypes.data_as(ctypes.POINTER(N.RtTensorDesc)), 1, 12)
+
+
+# ---- the C++ descriptor gatherer (host logic only; CPU tensors stand in with dev = -1) ----------
+def test_gatherer_writes_the_rows_the_python_loop_would():
+    from ramtorch_amd import _gather as G
+    g = G.module()
+    if g is None:
+        pytest.skip("gather helper not built")
+    n = 300
+    ps = [torch.nn.Parameter(torch.zeros(7 + i % 5, dtype=torch.bfloat16 if i % 2 else torch.float32)) for i in range(n)]
+    sts = [{"step": i % 3, "ema": torch.zeros_like(p), "ema_squared": torch.zeros_like(p, dtype=torch.float32)}
+           for i, p in enumerate(ps)]
+    for i, p in enumerate(ps):
+        if i % 7:
+            p.grad = torch.ones_like(p)  # torch only stores a gradient of the parameter's own dtype
+    sts[5] = {}                                                # state not initialised -> Python
+    sts[9]["ema"] = torch.zeros(3, dtype=torch.bfloat16)       # size mismatch -> Python
+    sts[10]["ema_squared"] = torch.zeros(4, 3).t()[:, :3]      # not contiguous -> Python
+    sts[11]["step"] = torch.tensor(4)                          # step is not a plain int -> Python
+    ps[12] = torch.nn.Parameter(torch.zeros(5, dtype=torch.float64))
+    ps[12].grad = torch.ones_like(ps[12])                      # fp64 gradient -> Python (downcast there)
+    sts[13]["ema"] = torch.zeros(ps[13].numel(), dtype=torch.int16)  # unsupported dtype -> Python
+    old = [st.get("step") for st in sts]
+    buf = np.zeros(n, F.DESC_DTYPE)
+    stat = np.full(n, 255, np.uint8)
+    rows, steps = g.gather_group(ps, sts, -1, buf.ctypes.data, n, stat.ctypes.data, 4, 100)
+    assert sorted(steps) == [1, 2, 3]
+    for i in (5, 9, 10, 11, 12, 13):
+        assert stat[i] == g.PYTHON and (sts[i].get("step") is old[i])
+    code = {torch.bfloat16: 0, torch.float32: 1, torch.float16: 2}
+    j = 0
+    for i, p in enumerate(ps):
+        if p.grad is None:
+            assert stat[i] == g.NO_GRAD and sts[i].get("step") == old[i]  # adamw.py:114: no step increment
+            continue
+        if stat[i] == g.PYTHON:
+            continue
+        d, st = buf[j], sts[i]
+        j += 1
+        assert stat[i] == g.WRITTEN and st["step"] == old[i] + 1
+        assert (d["p"], d["g"], d["m"], d["v"]) == (p.data_ptr(), p.grad.data_ptr(), st["ema"].data_ptr(),
+                                                    st["ema_squared"].data_ptr())
+        assert d["numel"] == p.numel() and d["tensor_id"] == 100 + i and d["step"] == st["step"]
+        assert d["scalars_idx"] == 4 + steps.index(st["step"])
+        assert (d["p_dtype"], d["g_dtype"], d["m_dtype"], d["v_dtype"]) == (code[p.dtype], code[p.grad.dtype],
+                                                                             code[p.dtype], 1)
+        assert d["host_mask"] == 0 and d["elem_offset"] == 0 and d["noise_p"] == 0 and d["row_mean"] == 0
+    assert j == rows
+    # capacity is respected: what does not fit is left to Python, untouched
+    old = [st.get("step") for st in sts]
+    rows2, _ = g.gather_group(ps, sts, -1, buf.ctypes.data, 10, stat.ctypes.data, 0, 0)
+    assert rows2 == 10 and int((stat == g.WRITTEN).sum()) == 10
+    assert sum(st.get("step") != o for st, o in zip(sts, old)) == 10
+    # a tensor subclass is never touched
+    class T(torch.Tensor):
+        pass
+    sub = torch.zeros(4).as_subclass(T)
+    rows3, _ = g.gather_group([sub], [{"step": 0, "ema": torch.zeros(4), "ema_squared": torch.zeros(4)}], -1,
+                              buf.ctypes.data, 10, stat.ctypes.data, 0, 0)
+    assert rows3 == 0 and stat[0] == g.PYTHON
