@@ -136,6 +136,32 @@ def test_optimizer_default_layout_cpu_params_and_pinned_states():
     assert all(p.is_pinned() for p in ps)  # params were updated in place
 
 
+def test_optimizer_plain_pageable_cpu_params():
+    """Plain (not pinned) CPU parameters and gradients, the third input kind the reference accepts:
+    the copies are staged by the runtime instead of going by DMA, results are the same."""
+    shapes = [(70_000,), (257, 31)]
+    ps, gs, refs = [], [], []
+    for i, shp in enumerate(shapes):
+        n = int(np.prod(shp))
+        p, g, _, _ = oracle.synth_inputs(n, 950 + i)
+        t = torch.nn.Parameter(host16(p, pin=False).view(shp))
+        assert not t.is_pinned()
+        ps.append(t)
+        gs.append(g)
+        refs.append([p.copy(), np.zeros(n, np.uint16), np.zeros(n, np.uint16)])
+    opt = ramtorch_amd.AdamW(ps, seed=22, stream_chunk_bytes=65_536, **HP0)
+    for step in (1, 2):
+        for p, g in zip(ps, gs):
+            p.grad = host16(g, pin=False).view(p.shape)
+        opt.step()
+        sco = oracle.scalars_from_hparams(step=step, **HP0)
+        for i, (p, g) in enumerate(zip(ps, gs)):
+            oracle.step_tensor(refs[i][0], g, refs[i][1], refs[i][2], sco, seed=22, step=step, tensor_id=i)
+            np.testing.assert_array_equal(bits16(p), refs[i][0], err_msg=f"step {step} param {i}")
+            np.testing.assert_array_equal(bits16(opt.state[p]["ema"]), refs[i][1])
+            np.testing.assert_array_equal(bits16(opt.state[p]["ema_squared"]), refs[i][2])
+
+
 def test_optimizer_gpu_params_with_default_cpu_states():
     n = 20_000
     p, g, _, _ = oracle.synth_inputs(n, 950)
