@@ -9,6 +9,7 @@ import atexit
 import ctypes
 import os
 import sys
+import threading
 import weakref
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -158,6 +159,9 @@ class Handle:
         self._h = ctypes.c_void_p()
         check(lib().rt_create(int(device), ctypes.byref(self._h)))
         self.device = int(device)
+        # ctypes drops the GIL during a call and an rt_handle is not re-entrant: calls on one handle
+        # from several Python threads (the main thread and autograd's hook threads) take turns.
+        self._lock = threading.RLock()
         _live_handles.add(self)
 
     @property
@@ -183,58 +187,72 @@ class Handle:
 
     # -- thin wrappers ---------------------------------------------------------
     def step_multi(self, descs, n, scalars, n_scalars, seed, noise_mode, d_clip_coef=None, d_skip=None, stream=0):
-        check(lib().rt_step_multi(self.ptr, descs, n, scalars, n_scalars, seed, noise_mode, d_clip_coef, d_skip,
-                                  stream))
+        with self._lock:
+            check(lib().rt_step_multi(self.ptr, descs, n, scalars, n_scalars, seed, noise_mode, d_clip_coef,
+                                      d_skip, stream))
 
     def step_streamed(self, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, stream=0):
-        check(lib().rt_step_streamed(self.ptr, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, stream))
+        with self._lock:
+            check(lib().rt_step_streamed(self.ptr, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems,
+                                         stream))
 
     def step_streamed_async(self, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, stream=0) -> int:
         """Enqueue only; returns the ticket of the call."""
         t = ctypes.c_uint64()
-        check(lib().rt_step_streamed_async(self.ptr, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems,
-                                           stream, ctypes.byref(t)))
+        with self._lock:
+            check(lib().rt_step_streamed_async(self.ptr, descs, n, scalars, n_scalars, seed, noise_mode,
+                                               chunk_elems, stream, ctypes.byref(t)))
         return t.value
 
     def streamed_wait(self) -> None:
-        check(lib().rt_streamed_wait(self.ptr))
+        with self._lock:
+            check(lib().rt_streamed_wait(self.ptr))
 
     def streamed_completed(self) -> int:
         t = ctypes.c_uint64()
-        check(lib().rt_streamed_completed(self.ptr, ctypes.byref(t)))
+        with self._lock:
+            check(lib().rt_streamed_completed(self.ptr, ctypes.byref(t)))
         return t.value
 
     def grad_norm(self, descs, n, inv_loss_scale, max_norm, d_out, stream=0):
-        check(lib().rt_grad_norm(self.ptr, descs, n, inv_loss_scale, max_norm, d_out, stream))
+        with self._lock:
+            check(lib().rt_grad_norm(self.ptr, descs, n, inv_loss_scale, max_norm, d_out, stream))
 
     def row_means(self, g, g_dtype, rows, row_len, inv_loss_scale, d_row_mean, stream=0):
-        check(lib().rt_row_means(self.ptr, g, g_dtype, rows, row_len, inv_loss_scale, d_row_mean, stream))
+        with self._lock:
+            check(lib().rt_row_means(self.ptr, g, g_dtype, rows, row_len, inv_loss_scale, d_row_mean, stream))
 
     def set_timing(self, enabled: bool) -> None:
-        check(lib().rt_set_timing(self.ptr, int(enabled)))
+        with self._lock:
+            check(lib().rt_set_timing(self.ptr, int(enabled)))
 
     def last_kernel_ms(self) -> float:
         ms = ctypes.c_float()
-        check(lib().rt_last_kernel_ms(self.ptr, ctypes.byref(ms)))
+        with self._lock:
+            check(lib().rt_last_kernel_ms(self.ptr, ctypes.byref(ms)))
         return ms.value
 
     def stream_probe(self, p, g, m, v, numel, reps=5, stream=0) -> float:
         """Mean ms per pass of the math-free traffic pattern (see rt_stream_probe)."""
         ms = ctypes.c_float()
-        check(lib().rt_stream_probe(self.ptr, p, g, m, v, numel, reps, ctypes.byref(ms), stream))
+        with self._lock:
+            check(lib().rt_stream_probe(self.ptr, p, g, m, v, numel, reps, ctypes.byref(ms), stream))
         return ms.value
 
     def streamed_timeline(self):
         """[(h2d_begin, h2d_end, d2h_begin, d2h_end), ...] in ms for the last timed streamed call."""
         n = ctypes.c_uint32()
-        check(lib().rt_streamed_timeline(self.ptr, None, 0, ctypes.byref(n)))
+        with self._lock:
+            check(lib().rt_streamed_timeline(self.ptr, None, 0, ctypes.byref(n)))
         buf = (ctypes.c_float * max(n.value, 1))()
-        check(lib().rt_streamed_timeline(self.ptr, buf, n.value, ctypes.byref(n)))
+        with self._lock:
+            check(lib().rt_streamed_timeline(self.ptr, buf, n.value, ctypes.byref(n)))
         return [tuple(buf[i:i + 4]) for i in range(0, n.value, 4)]
 
     def streamed_stats(self):
         out = (ctypes.c_double * 3)()
-        check(lib().rt_streamed_stats(self.ptr, out))
+        with self._lock:
+            check(lib().rt_streamed_stats(self.ptr, out))
         return {"bytes_h2d": out[0], "bytes_d2h": out[1], "seconds": out[2]}
 
 

@@ -555,12 +555,21 @@ class AdamW(Optimizer):
         is a number the pipeline writes into pinned host memory, so waiting for it never
         enters the runtime."""
         h = _handle(dev)
+        last_done, last_change = -1, time.monotonic()
         while True:
             done = h.streamed_completed()
             self._inflight = [x for x in self._inflight if not (x[0] == dev and x[1] <= done)]
             mine = [x for x in self._inflight if x[0] == dev]
             if len(mine) < self.max_inflight_calls and sum(x[2] for x in mine) <= self.max_inflight_bytes:
                 return
+            if done != last_done:
+                last_done, last_change = done, time.monotonic()
+            elif time.monotonic() - last_change > 60.0:
+                # no chunk has finished for a minute: fall back to a blocking wait, which
+                # either returns or raises the device error behind the stall
+                with torch.cuda.device(dev):
+                    h.streamed_wait()
+                last_change = time.monotonic()
             time.sleep(self._poll_seconds)
 
     def finish_early_steps(self) -> None:
