@@ -96,12 +96,18 @@ class AdamW(Optimizer):
         stream_chunk_bytes: bytes of bf16 per staged chunk of the host-resident path.
         loss_scale: gradients are divided by this inside the kernel.
         max_grad_norm: global L2 clip computed on the GPU before the update.
+        noise_source: "philox" (default) draws the rounding noise inside the kernel;
+            "reference" draws it the way the reference does -- three ``torch.randint``
+            tensors per parameter from generators seeded ``step + 42 / 69 / 420``
+            (adamw.py:10-21, 206-218) -- and feeds it to the kernel as explicit noise, so
+            that a run is bit-identical to ``ramtorch.AdamW`` under the same torch build.
+            A verification mode: it costs the three draws and their memory.
     """
 
     def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=1e-2, centralization=0,
                  chunk_size=64, dtype=torch.bfloat16, storage_device="cpu", *, seed: int = 0,
                  stream_chunk_bytes: int = 256 << 20, loss_scale: float = 1.0,
-                 max_grad_norm: Optional[float] = None):
+                 max_grad_norm: Optional[float] = None, noise_source: str = "philox"):
         defaults = dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay, centralization=centralization)
         super().__init__(params, defaults)
         self.chunk_size = chunk_size
@@ -111,6 +117,9 @@ class AdamW(Optimizer):
         self.stream_chunk_bytes = int(stream_chunk_bytes)
         self.loss_scale = float(loss_scale)
         self.max_grad_norm = max_grad_norm
+        if noise_source not in ("philox", "reference"):
+            raise ValueError(f"noise_source must be 'philox' or 'reference', got {noise_source!r}")
+        self.noise_source = noise_source
         self.last_grad_norm: Optional[torch.Tensor] = None  # [norm, clip_coef, found_inf bits, -] on the GPU
         self.fuse_in_backward = True      # the hook of make_post_accumulate_hook() is live
         self.max_inflight_bytes = 2 << 30  # gradients kept alive for updates still in flight (step_param)
@@ -267,6 +276,8 @@ class AdamW(Optimizer):
         recs = self._records()
         self.finish_early_steps()  # updates started from the backward hook must have landed
         early = self._stepped_early
+        if noise is None and getattr(self, "noise_source", "philox") == "reference":
+            noise = self._reference_noise(grads, early)
         scalars: List[N.RtScalars] = []
         scalar_key: Dict[tuple, int] = {}
         # plain lane: tensors wholly on one GPU, contiguous, nothing special -> columns only
@@ -422,6 +433,35 @@ class AdamW(Optimizer):
                 dst.copy_(tmp)
         early.clear()
         return loss
+
+    def _reference_noise(self, grads, early) -> dict:
+        """The reference's own rounding noise for every parameter about to step: a fresh
+        generator on the compute device seeded ``step + 42`` (param), ``+ 69`` (ema), ``+ 420``
+        (ema_squared) with the step count after the increment, ``randint(0, 65536)`` of the
+        parameter's shape (adamw.py:10-21, 177, 206-218).  Returned as int16 bit patterns."""
+        out = {}
+        for group in self.param_groups:
+            for p in group["params"]:
+                grad = grads.get(p, p.grad) if grads is not None else p.grad
+                if grad is None or (early and id(p) in early):
+                    continue
+                state = self.state[p]
+                if not state:
+                    self._init_state(p)
+                step = state["step"] + 1
+                dev = torch.device("cuda", _compute_device_index(p))
+                draws = []
+                for is_bf16, offset in ((p.dtype == torch.bfloat16, 42), (state["ema"].dtype == torch.bfloat16, 69),
+                                        (state["ema_squared"].dtype == torch.bfloat16, 420)):
+                    if not is_bf16:
+                        draws.append(None)  # written back with a plain copy_: no noise drawn (adamw.py:208,221)
+                        continue
+                    gen = torch.Generator(device=dev)
+                    gen.manual_seed(step + offset)
+                    r = torch.randint(low=0, high=(1 << 16), size=p.shape, dtype=torch.int32, device=dev, generator=gen)
+                    draws.append(r.to(torch.int16).view(-1))  # keeps the low 16 bits
+                out[p] = tuple(draws)
+        return out
 
     # -- updating one parameter as soon as its gradient exists --------------------------------
     def make_post_accumulate_hook(self):

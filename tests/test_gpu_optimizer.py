@@ -125,6 +125,31 @@ def test_other_param_and_state_dtypes_match_the_reference_op_sequence(p_dt, s_dt
             assert _nmis_any(st["ema_squared"], ref_v[i]) == 0, f"step {step} ema_squared {i}"
 
 
+@pytest.mark.parametrize("where", ["cuda", "cpu"])
+def test_reference_noise_mode_is_bit_identical_to_the_reference_step(where):
+    """noise_source="reference": the rounding noise is drawn exactly as adamw.py:10-21 does
+    (generators seeded step+42 / +69 / +420), so whole steps equal the reference's op
+    sequence drawing its own noise -- nothing is passed in from outside."""
+    shapes = [(64, 48), (1000,), (3, 5, 7), (8192 * 2 + 3,)]
+    ps, grads = _make_params(shapes, 1300, device="cuda")
+    if where == "cpu":
+        ps = [torch.nn.Parameter(p.detach().cpu().pin_memory()) for p in ps]
+    ref_p = [p.detach().clone().cuda() for p in ps]
+    opt = ramtorch_amd.AdamW(ps, lr=2e-3, storage_device=where, noise_source="reference", stream_chunk_bytes=32768)
+    ref_m = [torch.zeros_like(p) for p in ref_p]
+    ref_v = [torch.zeros_like(p) for p in ref_p]
+    for step in (1, 2, 3):
+        gmap = {p: (grads[i].float() * (1.0 + 0.3 * step)).bfloat16() for i, p in enumerate(ps)}
+        opt.step(grads=gmap)
+        torch.cuda.synchronize()
+        for i, p in enumerate(ps):
+            torch_ops.reference_step_ops(ref_p[i], gmap[p], ref_m[i], ref_v[i], lr=2e-3, betas=(0.9, 0.999), eps=1e-8,
+                                         weight_decay=1e-2, step=step, noise=None)
+            assert nmis(p.detach(), ref_p[i]) == 0, f"step {step} param {i}"
+            assert nmis(opt.state[p]["ema"], ref_m[i]) == 0, f"step {step} ema {i}"
+            assert nmis(opt.state[p]["ema_squared"], ref_v[i]) == 0, f"step {step} ema_squared {i}"
+
+
 def test_skipped_and_sparse_gradients():
     ps, grads = _make_params([(32, 8), (40,)], 200)
     opt = ramtorch_amd.AdamW(ps, storage_device="cuda")
