@@ -108,11 +108,14 @@ def test_other_param_and_state_dtypes_match_the_reference_op_sequence(p_dt, s_dt
     for step in (1, 2):
         noise, gmap = {}, {}
         for i, p in enumerate(ps):
-            gmap[p] = (grads[i].float() * (1.0 + 0.25 * step)).bfloat16()
+            # the gradient has the parameter's dtype and lives where the parameter lives, as autograd
+            # leaves it (fp64 and CPU gradients included: adamw.py:167 takes any float dtype, any device)
+            gmap[p] = (grads[i].float() * (1.0 + 0.25 * step)).to(p_dt)
+            p.grad = gmap[p].to(p.device)
             noise[p] = tuple(torch.randint(-32768, 32768, p.shape, dtype=torch.int16, device="cuda",
                                            generator=torch.Generator("cuda").manual_seed(step * 10 + i * 3 + k))
                              for k in range(3))
-        opt.step(noise=noise, grads=gmap)
+        opt.step(noise=noise)
         torch.cuda.synchronize()
         for i, p in enumerate(ps):
             st = opt.state[p]
