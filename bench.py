@@ -177,6 +177,8 @@ def main() -> int:
     ap.add_argument("--workload", default="llama8b", choices=["llama8b", "cfg0", "small", "mixed", "streamed", "hooked"])
     ap.add_argument("--layers", type=int, default=32, help="transformer layers of the Llama-shaped set")
     ap.add_argument("--stream-gb", type=float, default=48.2, help="upper bound on pinned host bytes (streamed)")
+    ap.add_argument("--state-placement", default="auto", choices=["auto", "plain"],
+                    help="AdamW(state_placement=...): 'auto' puts ema and ema_squared into different HBM regions")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pmc-calibrate", action="store_true",
                     help="also launch one plain elementwise kernel that reads 1 GiB and writes 1 GiB, so that "
@@ -199,7 +201,7 @@ def main() -> int:
     wl = args.workload
     first_step = 100
     noise = None
-    opt_kw = dict(storage_device="cuda", seed=1234)
+    opt_kw = dict(storage_device="cuda", seed=1234, state_placement=args.state_placement)
     bytes_per_elem = 14
     dtype_label = "f32"  # arithmetic type; storage is bf16 (or fp32 for the mixed layout)
     if wl == "llama8b":
@@ -220,7 +222,7 @@ def main() -> int:
         shapes = llama3_8b_shapes(args.layers)
         params, grads = build_resident(shapes, g_dtype=torch.float32, v_dtype=torch.float32, device=dev)
         state_dtype = torch.bfloat16
-        opt_kw.update(loss_scale=1024.0, max_grad_norm=1.0)
+        opt_kw.update(loss_scale=1024.0, max_grad_norm=1.0, ema_squared_dtype=torch.float32)
         bytes_per_elem = 24
     else:  # streamed / hooked
         shapes = llama3_8b_shapes(args.layers)
@@ -248,13 +250,9 @@ def main() -> int:
     for i, p in enumerate(params):
         st = opt.state[p]
         st["step"] = first_step - 1 - args.warmup
-        if wl not in ("streamed", "hooked"):
-            st["ema"] = fill_tensor(p.shape, "m", 1234 + 4 * i + 2, torch.bfloat16, dev)
-            vdt = torch.float32 if wl == "mixed" else torch.bfloat16
-            st["ema_squared"] = fill_tensor(p.shape, "v", 1234 + 4 * i + 3, vdt, dev)
-        else:
-            st["ema"].copy_(fill_tensor(p.shape, "m", 1234 + 4 * i + 2, torch.bfloat16, dev))
-            st["ema_squared"].copy_(fill_tensor(p.shape, "v", 1234 + 4 * i + 3, torch.bfloat16, dev))
+        # the states stay the tensors the optimizer allocated (and placed); only their contents are set
+        st["ema"].copy_(fill_tensor(p.shape, "m", 1234 + 4 * i + 2, torch.bfloat16, dev))
+        st["ema_squared"].copy_(fill_tensor(p.shape, "v", 1234 + 4 * i + 3, st["ema_squared"].dtype, dev))
     if wl == "cfg0":
         noise = {params[0]: tuple(torch.randint(-32768, 32768, (4096, 4096), dtype=torch.int16, device=dev,
                                                 generator=torch.Generator(dev).manual_seed(1234 + k))
@@ -313,14 +311,27 @@ def main() -> int:
                     "traffic": MEASURED_TRAFFIC_BYTES.get(wl) if args.layers == 32 else None,
                     "kernel": "sr_adamw_fast_kernel",
                     "kernel_ms": k_ms, "algorithmic_bytes_per_launch": upd_bytes}
-        # what the same traffic pattern reaches on this device with the arithmetic removed
+        # What the same traffic pattern reaches with the arithmetic removed (the all-bf16 pattern:
+        # 8 B read + 6 B written per element).  Where the arrays lie in HBM matters (see
+        # ramtorch_amd/placement.py), so it is measured twice: on four fresh buffers allocated
+        # side by side, and on the workload's own largest tensor (p, its gradient and its two
+        # states, where the optimizer placed them).  The probe overwrites what it runs on, which
+        # is why it comes last.
         n_probe = 1 << 30
         bufs = [torch.zeros(n_probe, dtype=torch.bfloat16, device=dev) for _ in range(4)]
         torch.cuda.synchronize()
         probe_ms = handle.stream_probe(*[b.data_ptr() for b in bufs], n_probe, reps=5)
-        roofline["pattern_ceiling_GBps"] = 14 * n_probe / (probe_ms * 1e-3) / 1e9
-        roofline["frac_of_pattern_ceiling"] = achieved / roofline["pattern_ceiling_GBps"] if wl in ("llama8b", "small") else None
+        roofline["pattern_ceiling_fresh_buffers_GBps"] = 14 * n_probe / (probe_ms * 1e-3) / 1e9
         del bufs
+        roofline["pattern_ceiling_GBps"] = roofline["pattern_ceiling_fresh_buffers_GBps"]
+        big = max(range(len(params)), key=lambda i: params[i].numel())
+        arrs = [params[big].data, grads[big], opt.state[params[big]]["ema"], opt.state[params[big]]["ema_squared"]]
+        n_own = min(a.numel() * a.element_size() // 2 for a in arrs) // 8192 * 8192
+        if n_own >= (1 << 24) and all(a.data_ptr() % 16 == 0 for a in arrs):
+            probe_ms = handle.stream_probe(*[a.data_ptr() for a in arrs], n_own, reps=5)
+            roofline["pattern_ceiling_GBps"] = 14 * n_own / (probe_ms * 1e-3) / 1e9
+        roofline["frac_of_pattern_ceiling"] = achieved / roofline["pattern_ceiling_GBps"] if wl in ("llama8b", "small") else None
+        roofline["state_placement"] = {"mode": args.state_placement, **(opt.state_placement_report or {})}
     else:
         if wl == "streamed":
             st = handle.streamed_stats()

@@ -147,9 +147,20 @@ struct KernelPair {
 
 template <int P, int G, int M, int V>
 static KernelPair pick_noise(int noise) {
-    if (noise == RT_NOISE_EXPLICIT)
-        return {sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_EXPLICIT>, sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_EXPLICIT>};
-    return {sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_PHILOX>, sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_PHILOX>};
+    // combinations with an fp32 array use the lane mapping that keeps every access contiguous across the wave
+    constexpr bool wide = P == RT_DT_F32 || G == RT_DT_F32 || M == RT_DT_F32 || V == RT_DT_F32;
+    if constexpr (wide) {
+        if (noise == RT_NOISE_EXPLICIT)
+            return {sr_adamw_fast_wide_kernel<P, G, M, V, RT_NOISE_EXPLICIT>,
+                    sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_EXPLICIT>};
+        return {sr_adamw_fast_wide_kernel<P, G, M, V, RT_NOISE_PHILOX>,
+                sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_PHILOX>};
+    } else {
+        if (noise == RT_NOISE_EXPLICIT)
+            return {sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_EXPLICIT>,
+                    sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_EXPLICIT>};
+        return {sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_PHILOX>, sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_PHILOX>};
+    }
 }
 template <int P, int G, int M>
 static KernelPair pick_v(int v, int noise) {

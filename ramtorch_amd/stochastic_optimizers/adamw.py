@@ -102,16 +102,27 @@ class AdamW(Optimizer):
             (adamw.py:10-21, 206-218) -- and feeds it to the kernel as explicit noise, so
             that a run is bit-identical to ``ramtorch.AdamW`` under the same torch build.
             A verification mode: it costs the three draws and their memory.
+        state_placement: "auto" (default) or "plain".  With GPU-resident states of at least
+            ``state_pool_min_bytes`` per kind, "auto" carves all ``ema`` tensors out of one
+            pool and all ``ema_squared`` tensors out of another and places the two pools in
+            different HBM regions, found by measurement at construction (see
+            ``ramtorch_amd/placement.py``; the outcome is in ``state_placement_report``).
+            "plain" allocates every state tensor on its own, as the reference does.
     """
 
     def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=1e-2, centralization=0,
                  chunk_size=64, dtype=torch.bfloat16, storage_device="cpu", *, seed: int = 0,
                  stream_chunk_bytes: int = 256 << 20, loss_scale: float = 1.0,
-                 max_grad_norm: Optional[float] = None, noise_source: str = "philox"):
+                 max_grad_norm: Optional[float] = None, noise_source: str = "philox",
+                 state_placement: str = "auto", state_pool_min_bytes: int = 1 << 30,
+                 ema_squared_dtype: Optional[torch.dtype] = None):
         defaults = dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay, centralization=centralization)
         super().__init__(params, defaults)
         self.chunk_size = chunk_size
         self.optim_state_dtype = dtype
+        # the reference keeps both states in one dtype; a wider second moment (bf16 ema, fp32
+        # ema_squared) is a common mixed layout and costs nothing extra in the kernel
+        self.ema_squared_dtype = dtype if ema_squared_dtype is None else ema_squared_dtype
         self.optim_state_device = storage_device
         self.seed = int(seed)
         self.stream_chunk_bytes = int(stream_chunk_bytes)
@@ -132,7 +143,15 @@ class AdamW(Optimizer):
         self._stepped_early = set()       # id(param) updated by step_param since the last step()
         self._inflight = []               # (device, ticket, bytes, tensors kept alive)
         self._early_batch = {}            # device -> [[entry, scalars, handed-over elements], ...], pending elements
+        if state_placement not in ("auto", "plain"):
+            raise ValueError(f"state_placement must be 'auto' or 'plain', got {state_placement!r}")
+        self.state_placement = state_placement
+        self.state_pool_min_bytes = int(state_pool_min_bytes)
+        self.state_placement_report = None
+        self._state_pools = {}            # "ema" / "ema_squared" -> byte pool; "slots": per parameter, in
+                                          # param_groups order: (offset in elements, numel) or None
         # eager state allocation, as adamw.py:84-104
+        self._allocate_pooled_states()
         for group in self.param_groups:
             for p in group["params"]:
                 if not self.state[p]:
@@ -145,6 +164,8 @@ class AdamW(Optimizer):
         self._desc_cache = {}
         self._state_lists = {}
         self.__dict__.setdefault("gather_min_tensors", 256)
+        self.__dict__.setdefault("_state_pools", {})
+        self.__dict__.setdefault("state_placement_report", None)
         self.__dict__.setdefault("_gather_bufs", {})
         self.__dict__.setdefault("_gather_stat", None)
 
@@ -169,13 +190,18 @@ class AdamW(Optimizer):
             self.seed = int(extra["seed"])
         saved_ids = [i for g in state_dict["param_groups"] for i in g["params"]]
         ours = [p for g in self.param_groups for p in g["params"]]
-        for idx, p in zip(saved_ids, ours):
+        for k_flat, (idx, p) in enumerate(zip(saved_ids, ours)):
             saved = state_dict["state"].get(idx)
             if saved is None:
                 continue
             st = self.state[p]
             for k in ("ema", "ema_squared"):
                 if k in saved and torch.is_tensor(saved[k]):
+                    slot = self._pool_view(k_flat, p, k)
+                    if slot is not None and slot.dtype == saved[k].dtype and slot.shape == saved[k].shape:
+                        slot.copy_(saved[k])   # keeps the placement chosen at construction
+                        st[k] = slot
+                        continue
                     t = saved[k].detach().to(device=self.optim_state_device).clone(
                         memory_format=torch.contiguous_format)
                     if self.optim_state_device == "cpu" and torch.cuda.is_available():
@@ -186,19 +212,75 @@ class AdamW(Optimizer):
         self._state_lists = {}
 
     # -- state ---------------------------------------------------------------------
-    def _new_state_tensor(self, p: torch.Tensor) -> torch.Tensor:
-        t = torch.zeros_like(p.data, dtype=self.optim_state_dtype, device=self.optim_state_device,
+    def _state_dtype(self, key: str) -> torch.dtype:
+        if key == "ema_squared":
+            return self.__dict__.get("ema_squared_dtype") or self.optim_state_dtype
+        return self.optim_state_dtype
+
+    def _new_state_tensor(self, p: torch.Tensor, key: str = "ema") -> torch.Tensor:
+        t = torch.zeros_like(p.data, dtype=self._state_dtype(key), device=self.optim_state_device,
                              memory_format=torch.contiguous_format)
         if self.optim_state_device == "cpu" and torch.cuda.is_available():
             # adamw.py:91-97 pins unconditionally; without a GPU there is nothing to pin for
             t = t.pin_memory()
         return t
 
+    def _allocate_pooled_states(self) -> None:
+        """GPU-resident states as views into two pools placed in different HBM regions
+        (``state_placement="auto"``).  Leaves ``self.state`` untouched when that does not
+        apply; ``_init_state`` then allocates tensor by tensor."""
+        if self.state_placement != "auto" or not torch.cuda.is_available():
+            return
+        try:
+            dev = torch.device(self.optim_state_device)
+        except (TypeError, RuntimeError):
+            return
+        if dev.type != "cuda":
+            return
+        if dev.index is None:
+            dev = torch.device("cuda", torch.cuda.current_device())
+        params = [p for g in self.param_groups for p in g["params"]]
+        esize = {k: torch.empty((), dtype=self._state_dtype(k)).element_size() for k in ("ema", "ema_squared")}
+        slots, total = [], 0      # slot offsets in elements (multiples of 256), the same in both pools
+        for p in params:
+            if self.state[p]:
+                slots.append(None)
+                continue
+            slots.append((total, p.numel()))
+            total += (p.numel() + 255) // 256 * 256
+        if total * min(esize.values()) < self.state_pool_min_bytes:
+            return
+        from .. import placement
+        N.lib()
+        with torch.cuda.device(dev):
+            pool_m, pool_v, report = placement.place_pair(_handle(dev.index), dev, total * esize["ema"],
+                                                          total * esize["ema_squared"])
+        self.state_placement_report = report
+        self._state_pools = {"ema": pool_m, "ema_squared": pool_v, "slots": slots}
+        for k, p in enumerate(params):
+            if slots[k] is None:
+                continue
+            st = self.state[p]
+            st["step"] = 0
+            st["ema"] = self._pool_view(k, p, "ema")
+            st["ema_squared"] = self._pool_view(k, p, "ema_squared")
+
+    def _pool_view(self, k: int, p: torch.Tensor, key: str) -> Optional[torch.Tensor]:
+        """The slot of the k-th parameter (param_groups order) in the pool of ``key`` as a
+        tensor of p's shape, or None when there is no such slot."""
+        pools = self.__dict__.get("_state_pools") or {}
+        slots = pools.get("slots") or []
+        if key not in pools or k >= len(slots) or slots[k] is None or slots[k][1] != p.numel():
+            return None
+        off, numel = slots[k]
+        es = torch.empty((), dtype=self._state_dtype(key)).element_size()
+        return pools[key][off * es:(off + numel) * es].view(self._state_dtype(key)).view(p.shape)
+
     def _init_state(self, p: torch.Tensor) -> None:
         state = self.state[p]
         state["step"] = 0
         state["ema"] = self._new_state_tensor(p)
-        state["ema_squared"] = self._new_state_tensor(p)
+        state["ema_squared"] = self._new_state_tensor(p, "ema_squared")
 
     def _tensor_ids(self) -> Dict[int, int]:
         ids: Dict[int, int] = {}

@@ -418,3 +418,61 @@ def test_gathered_step_equals_the_python_loop():
             assert nmis(oa.state[p]["ema"], ob.state[q]["ema"]) == 0, (step, i)
             assert nmis(oa.state[p]["ema_squared"], ob.state[q]["ema_squared"]) == 0, (step, i)
     assert max(oa.state[p]["step"] for p in a) == 3 and min(oa.state[p]["step"] for p in a) >= 2
+
+
+def test_pooled_state_placement_changes_nothing_but_addresses():
+    """state_placement="auto": ema and ema_squared are views into two pools (placed in different
+    HBM regions when the probe finds such a placement).  Results, state_dict and resume are the
+    same as with plain per-tensor states."""
+    shapes = [(9000, 8192), (70_000_003,), (4096,)]          # 143.7 M elements: 287 MB per pool
+    def make():
+        ps = []
+        for i, shp in enumerate(shapes):
+            g = torch.Generator("cuda").manual_seed(40 + i)
+            ps.append(torch.nn.Parameter((torch.randn(shp, device="cuda", generator=g) * 0.02).bfloat16(),
+                                         requires_grad=False))
+        return ps
+    a, b = make(), make()
+    oa = ramtorch_amd.AdamW(a, storage_device="cuda", seed=5, ema_squared_dtype=torch.float32,
+                            state_pool_min_bytes=64 << 20, **HP0)
+    ob = ramtorch_amd.AdamW(b, storage_device="cuda", seed=5, ema_squared_dtype=torch.float32, state_placement="plain",
+                            **HP0)
+    rep = oa.state_placement_report
+    assert rep is not None and rep["tries"] >= 1 and ob.state_placement_report is None
+    pm, pv = oa._state_pools["ema"], oa._state_pools["ema_squared"]
+    for p in a:
+        st = oa.state[p]
+        assert st["ema"].dtype == torch.bfloat16 and st["ema_squared"].dtype == torch.float32
+        assert st["ema"].shape == p.shape and st["ema"].is_contiguous() and st["ema"].data_ptr() % 256 == 0
+        assert pm.data_ptr() <= st["ema"].data_ptr() < pm.data_ptr() + pm.numel()
+        assert pv.data_ptr() <= st["ema_squared"].data_ptr() < pv.data_ptr() + pv.numel()
+        assert float(st["ema"].float().abs().max()) == 0.0 and float(st["ema_squared"].abs().max()) == 0.0
+    for step in (1, 2):
+        for i, (p, q) in enumerate(zip(a, b)):
+            g = torch.Generator("cuda").manual_seed(100 * step + i)
+            p.grad = (torch.randn(p.shape, device="cuda", generator=g) * 1e-3).bfloat16()
+            q.grad = p.grad.clone()
+        oa.step()
+        ob.step()
+    torch.cuda.synchronize()
+    for p, q in zip(a, b):
+        assert nmis(p.detach(), q.detach()) == 0
+        assert nmis(oa.state[p]["ema"], ob.state[q]["ema"]) == 0
+        assert _nmis_any(oa.state[p]["ema_squared"], ob.state[q]["ema_squared"]) == 0
+    # resume into a fresh optimizer: the loaded values land in its own pools
+    c = [torch.nn.Parameter(p.detach().clone(), requires_grad=False) for p in a]
+    oc = ramtorch_amd.AdamW(c, storage_device="cuda", seed=0, ema_squared_dtype=torch.float32,
+                            state_pool_min_bytes=64 << 20, **HP0)
+    oc.load_state_dict(copy.deepcopy(oa.state_dict()))
+    cm = oc._state_pools["ema"]
+    for p, r in zip(a, c):
+        assert oc.state[r]["step"] == 2 and oc.seed == 5
+        assert cm.data_ptr() <= oc.state[r]["ema"].data_ptr() < cm.data_ptr() + cm.numel()
+        assert nmis(oc.state[r]["ema"], oa.state[p]["ema"]) == 0
+        assert _nmis_any(oc.state[r]["ema_squared"], oa.state[p]["ema_squared"]) == 0
+        r.grad = p.grad.clone()
+    oa.step()
+    oc.step()
+    torch.cuda.synchronize()
+    for p, r in zip(a, c):
+        assert nmis(p.detach(), r.detach()) == 0

@@ -327,3 +327,15 @@ def test_gatherer_writes_the_rows_the_python_loop_would():
     rows3, _ = g.gather_group([sub], [{"step": 0, "ema": torch.zeros(4), "ema_squared": torch.zeros(4)}], -1,
                               buf.ctypes.data, 10, stat.ctypes.data, 0, 0)
     assert rows3 == 0 and stat[0] == g.PYTHON
+
+
+def test_state_layout_options_are_validated_and_harmless_on_cpu():
+    ps = [torch.nn.Parameter(torch.zeros(16, dtype=torch.bfloat16))]
+    with pytest.raises(ValueError, match="state_placement"):
+        ramtorch_amd.AdamW(ps, state_placement="somewhere")
+    with pytest.raises(ValueError, match="noise_source"):
+        ramtorch_amd.AdamW(ps, noise_source="dice")
+    opt = ramtorch_amd.AdamW(ps, ema_squared_dtype=torch.float32)  # bf16 ema, fp32 ema_squared
+    st = opt.state[ps[0]]
+    assert st["ema"].dtype == torch.bfloat16 and st["ema_squared"].dtype == torch.float32
+    assert opt.state_placement == "auto" and opt.state_placement_report is None and not opt._state_pools
