@@ -47,7 +47,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the update kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this script (scaled by the counters' readings for kernels of known size in the same runs).
-MEASURED_TRAFFIC_BYTES = {"llama8b": 112_546_570_807}
+MEASURED_TRAFFIC_BYTES = {"llama8b": 112_546_390_426}
 HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
 METRIC = "SR-AdamW step: params/sec + achieved HBM GB/s (% of peak), 8B bf16 set, 1 GPU"
 
