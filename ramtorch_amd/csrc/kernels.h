@@ -786,11 +786,47 @@ __device__ __forceinline__ float block_sum(float x, float* lds) {
 }
 
 // Sum of squares of one chunk of one gradient tensor (per-lane partial).
+// Whole chunk of an aligned gradient: every load is 16 bytes per lane and contiguous across the
+// wave whatever the element type (a sum does not care which lane gets which element), all loads
+// of the chunk are in flight together.
+template <int GDT>
+__device__ __forceinline__ float chunk_sumsq_full(const DevTensor& t, uint32_t chunk, float inv_loss_scale) {
+    constexpr int kLoads = (int)(kChunkElems * esize<GDT>() / 16 / kThreads);  // 4 (16-bit) or 8 (fp32)
+    const uint64_t base = t.g + (uint64_t)chunk * kChunkElems * esize<GDT>() + (uint64_t)threadIdx.x * 16;
+    u32x4 r[kLoads];
+#pragma unroll
+    for (int k = 0; k < kLoads; ++k) r[k] = ldg128(base + (uint64_t)k * (kThreads * 16));
+    float acc = 0.0f;
+#pragma unroll
+    for (int k = 0; k < kLoads; ++k) {
+        if constexpr (GDT == RT_DT_F32) {
+            const float x[4] = {u2f(r[k].x), u2f(r[k].y), u2f(r[k].z), u2f(r[k].w)};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float y = x[j] * inv_loss_scale;
+                acc = __builtin_fmaf(y, y, acc);
+            }
+        } else {
+            Raw8<GDT> raw;
+            raw.a = r[k];
+            float x[8];
+            decode<GDT>(raw, x);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float y = x[j] * inv_loss_scale;
+                acc = __builtin_fmaf(y, y, acc);
+            }
+        }
+    }
+    return acc;
+}
+
 template <int GDT>
 __device__ __forceinline__ float chunk_sumsq(const DevTensor& t, uint32_t chunk, float inv_loss_scale) {
     const uint64_t n = t.numel;
     const uint64_t chunk_base = (uint64_t)chunk * kChunkElems;
     const bool aligned = (t.g & 15u) == 0;
+    if (aligned && chunk_base + kChunkElems <= n) return chunk_sumsq_full<GDT>(t, chunk, inv_loss_scale);
     float acc = 0.0f;
 #pragma unroll 1
     for (int it = 0; it < kItersPerChunk; ++it) {
