@@ -309,7 +309,7 @@ def main() -> int:
         roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                     "frac": achieved / HBM_PEAK_GBPS,
                     "traffic": MEASURED_TRAFFIC_BYTES.get(wl) if args.layers == 32 else None,
-                    "kernel": "sr_adamw_fast_kernel",
+                    "kernel": "sr_adamw_fast_wide_kernel" if wl == "mixed" else "sr_adamw_fast_kernel",
                     "kernel_ms": k_ms, "algorithmic_bytes_per_launch": upd_bytes}
         # What the same traffic pattern reaches with the arithmetic removed (the all-bf16 pattern:
         # 8 B read + 6 B written per element).  Where the arrays lie in HBM matters (see
