@@ -352,6 +352,21 @@ def main() -> int:
             torch.cuda.synchronize()
             stream_info[f"pinned_{name}_peak_GBps"] = 8 * chunk / (time.perf_counter() - t1) / 1e9
         stream_info["h2d_frac_of_peak"] = stream_info["h2d_GBps"] / stream_info["pinned_h2d_peak_GBps"]
+        # both directions at once (what the pipeline does in steady state): two streams, one chunk each way
+        hbuf2 = torch.empty(chunk, dtype=torch.uint8).pin_memory()
+        dbuf2 = torch.empty(chunk, dtype=torch.uint8, device=dev)
+        s_up, s_down = torch.cuda.Stream(), torch.cuda.Stream()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(8):
+            with torch.cuda.stream(s_up):
+                dbuf.copy_(hbuf, non_blocking=True)
+            with torch.cuda.stream(s_down):
+                hbuf2.copy_(dbuf2, non_blocking=True)
+        torch.cuda.synchronize()
+        stream_info["pinned_duplex_peak_GBps_each_way"] = 8 * chunk / (time.perf_counter() - t1) / 1e9
+        stream_info["frac_of_duplex_peak"] = stream_info["d2h_GBps"] / stream_info["pinned_duplex_peak_GBps_each_way"]
+        del hbuf2, dbuf2
         if wl == "streamed":
             # per-chunk copy durations of one more step, from events the library records on its copy streams
             handle.set_timing(True)
