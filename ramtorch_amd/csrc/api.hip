@@ -788,7 +788,7 @@ static int streamed_wait(rt_handle* h) {
 }
 
 // Validates and enqueues the whole pipeline of one call; does not wait for it.
-static int streamed_enqueue(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
+static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
                             uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems, void* stream_,
                             bool trace, uint64_t* ticket_out) {
     if (!h) return fail(RT_EINVAL, "handle is NULL");
@@ -996,6 +996,30 @@ static int streamed_enqueue(rt_handle* h, const rt_tensor_desc* descs, uint32_t 
     if (ticket_out) *ticket_out = st.tickets_issued;
     if (trace) st.timeline.assign(4 * chunks.size(), 0.0f);
     return RT_OK;
+}
+
+// A call that fails after it has started to enqueue (a HIP error halfway through the chunk loop)
+// would leave the shared pipeline state -- buffer parity, buffer-free events -- out of step with
+// what the streams hold.  Drain the streams and start over from a clean state; the error of the
+// failed call is what the caller sees.
+static int streamed_enqueue(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
+                            uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems, void* stream_,
+                            bool trace, uint64_t* ticket_out) {
+    const int rc = streamed_enqueue_impl(h, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, stream_,
+                                         trace, ticket_out);
+    if (rc != RT_OK && h && h->st.ready) {
+        char saved[sizeof(g_err)];
+        memcpy(saved, g_err, sizeof(saved));
+        Streamed& st = h->st;
+        (void)hipStreamSynchronize(st.h2d);
+        (void)hipStreamSynchronize(st.comp);
+        (void)hipStreamSynchronize(st.d2h);
+        st.used_buf[0] = st.used_buf[1] = false;
+        st.pending = false;
+        for (auto& r : st.ring) r.in_flight = false;
+        memcpy(g_err, saved, sizeof(saved));
+    }
+    return rc;
 }
 
 int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
