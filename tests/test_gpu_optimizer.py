@@ -476,3 +476,61 @@ def test_pooled_state_placement_changes_nothing_but_addresses():
     torch.cuda.synchronize()
     for p, r in zip(a, c):
         assert nmis(p.detach(), r.detach()) == 0
+
+
+def test_random_parameter_sets_match_the_oracle():
+    """Seeded random optimizer-level cases: 1 to 300 tensors, GPU / pinned / pageable parameters,
+    GPU or host states, one or two groups, skipped gradients, C++ gatherer on or off, three steps."""
+    rng = np.random.default_rng(77)
+
+    def t16(a, where, pin):
+        t = torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16)
+        if where == "cuda":
+            return t.cuda()
+        return t.pin_memory() if pin else t
+
+    hp = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
+    hp2 = dict(lr=3e-4, betas=(0.8, 0.99), eps=1e-8, weight_decay=0.0)
+    for case in range(40):
+        k = int(rng.choice([1, 3, 17, 40, 300]))
+        p_where, s_where = str(rng.choice(["cuda", "cpu"])), str(rng.choice(["cuda", "cpu"]))
+        pin = bool(rng.random() < 0.7)
+        seed = int(rng.integers(0, 1 << 40))
+        lens = [max(1, int(x)) for x in np.exp(rng.uniform(0, np.log(30000), k))]
+        if rng.random() < 0.3:
+            lens[0] = 8192 * int(rng.integers(1, 5))
+        ps, ref = [], []
+        for i, n in enumerate(lens):
+            p, _, _, _ = oracle.synth_inputs(n, seed % 1000 + i)
+            shape = (n,) if n % 4 or rng.random() < 0.5 else (n // 4, 4)
+            ps.append(torch.nn.Parameter(t16(p, p_where, pin).view(shape), requires_grad=False))
+            ref.append([p.copy(), np.zeros(n, np.uint16), np.zeros(n, np.uint16), 0])
+        cut = k if k < 3 or rng.random() < 0.5 else int(rng.integers(1, k))
+        groups = [{"params": ps[:cut]}] + ([{"params": ps[cut:], **hp2}] if cut < k else [])
+        opt = ramtorch_amd.AdamW(groups, storage_device=s_where, seed=seed,
+                                 stream_chunk_bytes=int(rng.choice([4096, 65536, 1 << 20])), **hp)
+        opt.gather_min_tensors = int(rng.choice([1, 10 ** 9]))
+        for step in (1, 2, 3):
+            grads = []
+            for i, p in enumerate(ps):
+                if rng.random() < 0.15:
+                    p.grad = None
+                    grads.append(None)
+                    continue
+                _, g, _, _ = oracle.synth_inputs(lens[i], seed % 1000 + 7 * i + step)
+                p.grad = t16(g, p_where, False).view(p.shape)
+                grads.append(g)
+            opt.step()
+            torch.cuda.synchronize()
+            for i, p in enumerate(ps):
+                r = ref[i]
+                if grads[i] is not None:
+                    r[3] += 1
+                    sc = oracle.scalars_from_hparams(step=r[3], **(hp if i < cut else hp2))
+                    oracle.step_tensor(r[0], grads[i], r[1], r[2], sc, seed=seed, step=r[3], tensor_id=i)
+                st = opt.state[p]
+                what = f"case {case} ({k} tensors, params {p_where}, states {s_where}) tensor {i} step {step}"
+                assert st["step"] == r[3], what
+                assert int((bits16(p) != r[0]).sum()) == 0, what
+                assert int((bits16(st["ema"]) != r[1]).sum()) == 0, what
+                assert int((bits16(st["ema_squared"]) != r[2]).sum()) == 0, what

@@ -367,3 +367,39 @@ def test_bad_arguments_are_rejected(handle):
     e.tensor_id = 1 << 30
     with pytest.raises(N.NativeError, match="tensor_id"):
         F.step_resident(handle, [e], [F.make_scalars(step=1, **HP0)], seed=0, explicit_noise=False)
+
+
+# ---- seeded random cases: sizes, dtypes, hyper-parameters, steps, noise modes, scaling -----------------
+def test_random_cases_match_the_oracle(handle):
+    rng = np.random.default_rng(20240)
+    dts = [oracle.DT_BF16, oracle.DT_F32, oracle.DT_F16, oracle.DT_F64]
+
+    def conv(a, dt, scale=1.0):
+        f = oracle.bf16_to_f32(a) * np.float32(scale)
+        if dt == oracle.DT_F32:
+            return (f * np.float32(1.0009765625)).astype(np.float32)
+        if dt == oracle.DT_F16:
+            return f.astype(np.float16).view(np.uint16)
+        if dt == oracle.DT_F64:
+            return f.astype(np.float64) * (1.0 + 2.0 ** -30)
+        return a
+
+    for case in range(400):
+        n = max(1, int(rng.choice([rng.integers(1, 64), rng.integers(1, 9000), rng.integers(8000, 70000),
+                                   8192 * rng.integers(1, 6) + rng.integers(-9, 9)])))
+        p_dt, m_dt, v_dt = (int(rng.choice(dts, p=[0.55, 0.25, 0.1, 0.1])) for _ in range(3))
+        g_dt = int(rng.choice(dts[:3], p=[0.5, 0.35, 0.15]))
+        hp = dict(lr=float(10 ** rng.uniform(-5, -1)),
+                  betas=(float(rng.choice([0.0, 0.5, 0.9, 0.95])), float(rng.choice([0.9, 0.99, 0.999, 0.9999]))),
+                  eps=float(rng.choice([1e-8, 1e-6, 1e-12])), weight_decay=float(rng.choice([0.0, 0.01, 0.1])))
+        ls = float(rng.choice([1.0, 1.0, 1024.0, 65536.0]))
+        if g_dt == oracle.DT_F16:
+            ls = min(ls, 1024.0)
+        p, g, m, v = oracle.synth_inputs(n, int(rng.integers(0, 1 << 30)))
+        kw = dict(hp=hp, step=int(rng.choice([1, 2, 10, 1000, 123456])), seed=int(rng.integers(0, 1 << 62)),
+                  tensor_id=int(rng.integers(0, 1 << 20)), p_dtype=p_dt, g_dtype=g_dt, m_dtype=m_dt, v_dtype=v_dt,
+                  inv_loss_scale=1.0 / ls, clip_coef=None if rng.random() < 0.7 else float(rng.uniform(0.01, 1.0)),
+                  noise=oracle.synth_noise(n, int(rng.integers(0, 1 << 30))) if rng.random() < 0.4 else None,
+                  debug=bool(rng.random() < 0.5))
+        got, want, dbg, pre = run_both(handle, conv(p, p_dt), conv(g, g_dt, ls), conv(m, m_dt), conv(v, v_dt), **kw)
+        assert_same(got, want, dbg, pre, f"random case {case}: n={n} dtypes={(p_dt, g_dt, m_dt, v_dt)}")
