@@ -214,8 +214,12 @@ int rt_last_kernel_ms(rt_handle* h, float* ms);
  * returns the mean milliseconds per pass.  14 * numel / time is the rate this
  * access pattern can reach on the device: the practical ceiling the update
  * kernel is compared with.  The arrays are bf16-sized scratch of `numel`
- * elements (a multiple of 8192), 16-byte aligned; p, m, v are overwritten.
- * Blocks until done.
+ * elements (a multiple of 8192), 16-byte aligned; p, m, v are overwritten
+ * (each with itself xor g, so arrays of zeros stay zeros).  Blocks until done.
+ * The rate depends on where the four arrays lie in HBM (about 5.7 TB/s on
+ * MI355X with all of them in one region, 6.4 TB/s with one written array in
+ * another); callers that own their allocations can use this to choose a
+ * placement, as the Python optimizer does for its states.
  */
 int rt_stream_probe(rt_handle* h, void* p, const void* g, void* m, void* v, uint64_t numel, int reps,
                     float* ms_out, void* stream);
