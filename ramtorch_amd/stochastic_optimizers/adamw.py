@@ -42,14 +42,17 @@ def _compute_device_index(p: torch.Tensor) -> int:
     return torch.cuda.current_device()
 
 
-def copy_stochastic_(target: torch.Tensor, source: torch.Tensor, seed=0, *, noise: Optional[torch.Tensor] = None):
+def copy_stochastic_(target: torch.Tensor, source: torch.Tensor, seed=0, *, noise: Optional[torch.Tensor] = None,
+                     reference_noise: bool = False):
     """Stochastically round fp32 ``source`` into bf16 ``target`` (adamw.py:6-30):
     add 16 random bits below the bf16 mantissa, keep the high half.
 
     The reference draws the bits with ``torch.randint`` from a generator seeded
     with ``seed``; here they come from Philox4x32-10 keyed by ``seed`` (or from
-    ``noise``, an int16 tensor, for reproducible tests).  Both tensors must be
-    contiguous GPU tensors; a CPU ``target`` is filled through a GPU temporary.
+    ``noise``, an int16 tensor, for reproducible tests).  With ``reference_noise`` the
+    bits are drawn exactly as the reference draws them (adamw.py:10-21), which makes the
+    result bit-identical to the reference's under the same torch build.  Both tensors must
+    be contiguous GPU tensors; a CPU ``target`` is filled through a GPU temporary.
     """
     if source.dtype != torch.float32 or target.dtype != torch.bfloat16:
         raise TypeError("copy_stochastic_ rounds float32 -> bfloat16")
@@ -63,6 +66,11 @@ def copy_stochastic_(target: torch.Tensor, source: torch.Tensor, seed=0, *, nois
         dst = target if (target.is_cuda and target.is_contiguous()) else torch.empty(
             target.shape, dtype=torch.bfloat16, device=source.device)
         nz = None
+        if noise is None and reference_noise:
+            gen = torch.Generator(device=source.device)
+            gen.manual_seed(int(seed))
+            noise = torch.randint(low=0, high=(1 << 16), size=source.shape, dtype=torch.int32, device=source.device,
+                                  generator=gen).to(torch.int16)  # keeps the low 16 bits
         if noise is not None:
             if noise.dtype not in (torch.int16, torch.uint16) or noise.numel() != source.numel():
                 raise ValueError("noise must be an int16 tensor of source's size")

@@ -369,6 +369,13 @@ def test_copy_stochastic():
     cpu_tgt = torch.empty(n, dtype=torch.bfloat16)
     ramtorch_amd.copy_stochastic_(cpu_tgt, src, seed=42)
     assert nmis(cpu_tgt, tgt.cpu()) == 0
+    # the reference's own draw (adamw.py:10-21): a fresh generator seeded with `seed`
+    src2 = src.view(-1)[:100_000].view(250, 400)
+    tgt2 = torch.empty(250, 400, dtype=torch.bfloat16, device="cuda")
+    ramtorch_amd.copy_stochastic_(tgt2, src2, seed=77, reference_noise=True)
+    ref2 = torch.empty_like(tgt2)
+    torch_ops.sr_write_(ref2, src2, torch_ops.draw_noise(src2.shape, 77, src2.device))
+    assert nmis(ref2, tgt2) == 0
 
 
 def test_gathered_step_equals_the_python_loop():
