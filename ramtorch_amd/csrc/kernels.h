@@ -1,9 +1,11 @@
 // Device code of the stochastic-rounding AdamW step for gfx950 (wave64).
 //
 // The step is HBM-bound (14 bytes and ~25 flops per all-bf16 element), so the
-// kernels are plain vector code: 128-bit global loads and stores, fp32 math in
-// registers, a counter-based Philox4x32-10 for the rounding noise.  No LDS and
-// no MFMA in the update; wavefront reductions only in the norm / row-mean passes.
+// kernels are plain vector code: 128-bit global loads and stores (64-bit ones
+// for 16-bit arrays in the layout with fp32 arrays), each instruction
+// contiguous across the wave, fp32 math in registers, a counter-based
+// Philox4x32-10 for the rounding noise.  No LDS and no MFMA in the update;
+// wavefront reductions only in the norm / row-mean passes.
 //
 // Floating-point contraction is switched off for the whole file: the rounding
 // sequence of every operation is part of the contract (it has to reproduce
