@@ -165,17 +165,40 @@ class AdamW(Optimizer):
                 if not self.state[p]:
                     self._init_state(p)
 
+    # torch's Optimizer pickles only defaults / state / param_groups; everything this class adds
+    # to configure itself travels in one extra entry, so that copies and unpickled optimizers step.
+    _CONFIG_DEFAULTS = dict(chunk_size=64, optim_state_dtype=torch.bfloat16, ema_squared_dtype=None,
+                            optim_state_device="cpu", seed=0, stream_chunk_bytes=256 << 20, loss_scale=1.0,
+                            max_grad_norm=None, noise_source="philox", fuse_in_backward=True,
+                            max_inflight_bytes=2 << 30, max_inflight_calls=2, _poll_seconds=0.0002,
+                            gather_min_tensors=256, state_placement="auto", state_pool_min_bytes=1 << 30)
+
+    def __getstate__(self):
+        st = dict(super().__getstate__())
+        st["ramtorch_amd_config"] = {k: getattr(self, k, d) for k, d in self._CONFIG_DEFAULTS.items()}
+        return st
+
     def __setstate__(self, state):
-        # load_state_dict (and unpickling) replace self.state wholesale: drop everything derived from it
+        # Called when unpickling and by load_state_dict (which replaces self.state wholesale):
+        # drop everything derived from the state, keep or restore the configuration.
+        state = dict(state)
+        config = state.pop("ramtorch_amd_config", None)
         super().__setstate__(state)
+        if config:
+            self.__dict__.update(config)
+        for k, d in self._CONFIG_DEFAULTS.items():
+            self.__dict__.setdefault(k, d)
+        if self.__dict__.get("ema_squared_dtype") is None:
+            self.ema_squared_dtype = self.optim_state_dtype
         self._recs = None
         self._desc_cache = {}
         self._state_lists = {}
-        self.__dict__.setdefault("gather_min_tensors", 256)
-        self.__dict__.setdefault("_state_pools", {})
-        self.__dict__.setdefault("state_placement_report", None)
-        self.__dict__.setdefault("_gather_bufs", {})
-        self.__dict__.setdefault("_gather_stat", None)
+        for k, d in (("_state_pools", {}), ("state_placement_report", None), ("_gather_bufs", {}),
+                     ("_gather_stat", None), ("last_grad_norm", None)):
+            self.__dict__.setdefault(k, d)
+        for k, make in (("_stepped_early", set), ("_inflight", list), ("_early_batch", dict)):
+            if k not in self.__dict__:
+                self.__dict__[k] = make()
 
     def state_dict(self):
         """Same layout as the reference (``state`` with ``step / ema / ema_squared`` per

@@ -541,3 +541,23 @@ def test_random_parameter_sets_match_the_oracle():
                 assert int((bits16(p) != r[0]).sum()) == 0, what
                 assert int((bits16(st["ema"]) != r[1]).sum()) == 0, what
                 assert int((bits16(st["ema_squared"]) != r[2]).sum()) == 0, what
+
+
+def test_deepcopied_optimizer_steps_like_the_original():
+    ps, grads = _make_params([(300,), (16, 16)], 1500)
+    opt = ramtorch_amd.AdamW(ps, storage_device="cuda", seed=9, **HP0)
+    for p, g in zip(ps, grads):
+        p.grad = g
+    opt.step()
+    twin = copy.deepcopy(opt)          # copies parameters, states and the configuration
+    qs = twin.param_groups[0]["params"]
+    assert twin.seed == 9 and all(q is not p for p, q in zip(ps, qs))
+    for q, g in zip(qs, grads):
+        q.grad = g.clone()
+    opt.step()
+    twin.step()
+    torch.cuda.synchronize()
+    for p, q in zip(ps, qs):
+        assert nmis(p.detach(), q.detach()) == 0
+        assert nmis(opt.state[p]["ema"], twin.state[q]["ema"]) == 0
+        assert opt.state[p]["step"] == twin.state[q]["step"] == 2

@@ -338,3 +338,22 @@ def test_state_layout_options_are_validated_and_harmless_on_cpu():
     st = opt.state[ps[0]]
     assert st["ema"].dtype == torch.bfloat16 and st["ema_squared"].dtype == torch.float32
     assert opt.state_placement == "auto" and opt.state_placement_report is None and not opt._state_pools
+
+
+def test_copies_and_unpickled_optimizers_keep_their_configuration():
+    import copy
+    import pickle
+    ps = [torch.nn.Parameter(torch.zeros(16, dtype=torch.bfloat16))]
+    opt = ramtorch_amd.AdamW(ps, seed=7, loss_scale=4.0, max_grad_norm=1.5, noise_source="reference",
+                             ema_squared_dtype=torch.float32, state_placement="plain", chunk_size=3)
+    opt.max_inflight_calls = 5
+    for other in (copy.deepcopy(opt), pickle.loads(pickle.dumps(opt))):
+        assert (other.seed, other.loss_scale, other.max_grad_norm, other.noise_source) == (7, 4.0, 1.5, "reference")
+        assert other.ema_squared_dtype == torch.float32 and other.optim_state_dtype == torch.bfloat16
+        assert other.state_placement == "plain" and other.chunk_size == 3 and other.max_inflight_calls == 5
+        assert other._stepped_early == set() and other._inflight == [] and other._recs is None
+        q = other.param_groups[0]["params"][0]
+        assert other.state[q]["ema_squared"].dtype == torch.float32 and other.state[q]["step"] == 0
+    # load_state_dict goes through __setstate__ too and must leave the live configuration alone
+    opt.load_state_dict(copy.deepcopy(opt.state_dict()))
+    assert opt.max_inflight_calls == 5 and opt.loss_scale == 4.0
