@@ -157,14 +157,17 @@ def cpu_baseline(sample_elems: int = 4096 * 4096):
 # ---- GPU workloads ----------------------------------------------------------------------------
 def build_resident(shapes, *, g_dtype, v_dtype, device, seed=1234):
     import torch
+    # parameters first, gradients afterwards: the order a framework allocates them in (model
+    # construction, then the backward pass), so a parameter and its gradient are not neighbours
     params, grads = [], []
     for i, shp in enumerate(shapes):
-        p = torch.nn.Parameter(fill_tensor(shp, "p", seed + 4 * i, torch.bfloat16, device), requires_grad=False)
+        params.append(torch.nn.Parameter(fill_tensor(shp, "p", seed + 4 * i, torch.bfloat16, device),
+                                         requires_grad=False))
+    for i, shp in enumerate(shapes):
         g = fill_tensor(shp, "g", seed + 4 * i + 1, torch.float32 if g_dtype == torch.float32 else torch.bfloat16,
                         device)
         if g_dtype == torch.float32:
             g.mul_(1024.0)
-        params.append(p)
         grads.append(g)
     return params, grads
 
