@@ -1,6 +1,7 @@
 """Where the optimizer states sit in HBM.
 
-Measured on MI355X (288 GiB as three regions of roughly 92 GiB in physical address order): the
+Measured on MI355X (288 GiB as three regions of 96 GiB in physical address order; ``python -m
+ramtorch_amd.placement`` prints the map): the
 update's traffic -- four arrays read, three of them written in place -- runs at about 5.7 TB/s
 when p, ema and ema_squared all lie in one region and at about 6.4 TB/s as soon as one of the
 *written* arrays lies in another region; where the read-only gradient lies makes no difference.
@@ -104,3 +105,43 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
     torch.cuda.empty_cache()
     report["seconds"] = time.monotonic() - t0
     return a, b, report
+
+
+def _device_map(block_gib: int = 2, reserve_gib: int = 6) -> None:
+    """``python -m ramtorch_amd.placement``: maps how the update's traffic pattern runs depending on
+    where its four arrays lie.  Allocates nearly all free memory of the current GPU in blocks (memory
+    handed out block after block follows in physical address order) and probes combinations of blocks."""
+    from .stochastic_optimizers.adamw import _handle
+
+    dev = torch.device("cuda", torch.cuda.current_device())
+    handle = _handle(dev.index)
+    free, total = torch.cuda.mem_get_info(dev)
+    block = block_gib * GIB
+    n_blocks = int((free - reserve_gib * GIB) // block)
+    n = block // 2  # bf16 elements per block
+    blocks = [torch.empty(block, dtype=torch.uint8, device=dev) for _ in range(n_blocks)]
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def probe(idx, reps=3):
+        ms = handle.stream_probe(*(blocks[i].data_ptr() for i in idx), n, reps=reps, stream=stream)
+        return 14.0 * n / ms / 1e6
+
+    print(f"{torch.cuda.get_device_name(dev)}: {total / GIB:.0f} GiB, {n_blocks} blocks of {block_gib} GiB; "
+          "GB/s of 8 B read + 6 B written per element (p, g, ema, ema_squared; p, ema, ema_squared written)")
+    print("\n1. four neighbouring blocks (p, g, ema, ema_squared = blocks b .. b+3):")
+    print("   " + "  ".join(f"{b * block_gib}GiB:{probe((b, b + 1, b + 2, b + 3)):.0f}" for b in range(0, n_blocks - 3, 4)))
+    for base in (0, n_blocks // 2):
+        print(f"\n2. p, g, ema at blocks {base}..{base + 2}; ema_squared at block k (GiB into the allocation order : GB/s):")
+        ks = [k for k in range(0, n_blocks, 3) if not base <= k <= base + 2]
+        print("   " + "  ".join(f"{k * block_gib}:{probe((base, base + 1, base + 2, k)):.0f}" for k in ks))
+    a, b, c = 0, n_blocks // 2, n_blocks - 8
+    where = {"A": a, "B": b, "C": c}
+    print(f"\n3. which array has to move (A = block {a}.., B = block {b}.., C = block {c}..; order p g ema ema_squared):")
+    for pat in ("AAAA", "BBBB", "CCCC", "ABAA", "AAAB", "AABA", "BAAA", "AABB", "ABAB", "ABBA", "ABBB", "AABC", "ABCA", "ABCC"):
+        idx = tuple(where[r] + j for j, r in enumerate(pat))
+        print(f"   {pat}  {probe(idx, 5):.0f}")
+
+
+if __name__ == "__main__":
+    _device_map()
