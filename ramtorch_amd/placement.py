@@ -28,37 +28,48 @@ _MIN_ELEMS = 1 << 22     # below 8 MB per array the probe says little
 _MAX_ELEMS = 1 << 27     # 256 MB per array is plenty
 
 
-def split_probe(handle: N.Handle, a: torch.Tensor, b: torch.Tensor) -> Optional[Tuple[float, float]]:
-    """(GB/s with p, g, ema, ema_squared all inside ``a``, GB/s with ema_squared in ``b`` instead),
-    or None when the buffers are too small to tell.  ``a`` and ``b`` are 1-D GPU byte buffers."""
+def split_probe(handle: N.Handle, a: torch.Tensor, b: torch.Tensor):
+    """[(GB/s with p, g, ema, ema_squared all inside ``a``, GB/s with ema_squared in ``b`` instead), ...]
+    at the beginning, middle and end of the two buffers, or None when they are too small to tell.
+    ``a`` and ``b`` are 1-D GPU byte buffers of which corresponding parts will be used together (slot
+    k of one pool with slot k of the other): a pool that straddles a region boundary shows the gain
+    at some positions only."""
     na, nb = a.numel() * a.element_size() // 2, b.numel() * b.element_size() // 2
     n = min(na // 4, nb, _MAX_ELEMS)
     n -= n % _CHUNK
     if n < _MIN_ELEMS or (a.data_ptr() | b.data_ptr()) & 15:
         return None
     stream = torch.cuda.current_stream(a.device).cuda_stream
-    pa = [a.data_ptr() + 2 * n * k for k in range(4)]
-    with torch.cuda.device(a.device):
-        same = handle.stream_probe(pa[0], pa[1], pa[2], pa[3], n, reps=5, stream=stream)
-        cross = handle.stream_probe(pa[0], pa[1], pa[2], b.data_ptr(), n, reps=5, stream=stream)
     gb = 14.0 * n / 1e6
-    return gb / same, gb / cross
+    out = []
+    with torch.cuda.device(a.device):
+        for frac in (0.0, 0.5, 1.0):
+            # the same relative position in both pools; in `a` four consecutive pieces are needed
+            oa = int((na - 4 * n) * frac) // _CHUNK * _CHUNK
+            ob = int((nb - n) * frac) // _CHUNK * _CHUNK
+            pa = [a.data_ptr() + 2 * (oa + n * k) for k in range(4)]
+            same = gb / handle.stream_probe(pa[0], pa[1], pa[2], pa[3], n, reps=3, stream=stream)
+            cross = gb / handle.stream_probe(pa[0], pa[1], pa[2], b.data_ptr() + 2 * ob, n, reps=3, stream=stream)
+            out.append((same, cross))
+    return out
 
 
 def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: int, *,
                min_gain: float = 1.05, filler_bytes: int = 2 * GIB, step_bytes: int = 16 * GIB,
-               max_filler_bytes: int = 160 * GIB, max_seconds: float = 20.0,
+               max_filler_bytes: int = 112 * GIB, max_seconds: float = 8.0,
                log: Optional[Callable[[str], None]] = None):
-    """Two zeroed byte pools on ``device`` such that arrays in the second are, if it can be
-    arranged, in another HBM region than arrays in the first.  Returns (pool_a, pool_b, report).
+    """Two zeroed byte pools on ``device`` such that arrays in the second are, as far as it can be
+    arranged, in another HBM region than the corresponding arrays in the first.  Returns
+    (pool_a, pool_b, report).
 
-    The second pool is first allocated right after the first.  If the probe shows no gain,
-    filler blocks are allocated (memory the driver hands out in moderate blocks follows in
-    physical address order; one huge block does not) and after every ``step_bytes`` of them a
-    new candidate for the second pool is allocated and probed, until one shows the gain, or
-    ``max_filler_bytes`` (regions are smaller than that), free memory or ``max_seconds`` run
-    out.  Fillers and rejected candidates are released again and ``torch.cuda.empty_cache()``
-    returns them to the driver, which also drops whatever else torch had cached."""
+    The second pool is first allocated right after the first.  Unless the probe shows the gain
+    (mean over the beginning, middle and end of the pools), filler blocks are allocated (memory
+    the driver hands out in moderate blocks follows in physical address order; one huge block
+    does not) and after every ``step_bytes`` of them a new candidate for the second pool is
+    allocated and probed, until one shows the gain, or ``max_filler_bytes`` (a region is 96 GiB),
+    free memory or ``max_seconds`` run out; the candidate with the best mean rate is kept.
+    Fillers and the other candidates are released again and ``torch.cuda.empty_cache()`` returns
+    them to the driver, which also drops whatever else torch had cached."""
     import time
 
     def zeros(nbytes):
@@ -67,18 +78,21 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
     t0 = time.monotonic()
     report = {"placed": False, "filler_GiB": 0.0, "same_GBps": None, "cross_GBps": None, "tries": 0, "seconds": 0.0}
     a = zeros(bytes_a)
-    b = zeros(bytes_b)
-    res = split_probe(handle, a, b)
+    best = zeros(bytes_b)
+    res = split_probe(handle, a, best)
     if res is None:
-        return a, b, report
-    report.update(same_GBps=res[0], cross_GBps=res[1], tries=1)
-    if res[1] >= min_gain * res[0]:
-        report.update(placed=True, seconds=time.monotonic() - t0)
-        return a, b, report
-    held, filled = [], 0          # fillers and rejected candidates
-    chosen = None
+        return a, best, report
+
+    def summary(r):
+        same = sum(x[0] for x in r) / len(r)
+        cross = sum(x[1] for x in r) / len(r)
+        return same, cross, cross >= min_gain * same
+
+    same, cross, full = summary(res)
+    report.update(same_GBps=same, cross_GBps=cross, tries=1, placed=full)
+    held, filled = [], 0          # fillers and candidates that lost
     try:
-        while chosen is None:
+        while not report["placed"]:
             free, _ = torch.cuda.mem_get_info(device)
             if (filled + step_bytes > max_filler_bytes or step_bytes + bytes_b + 4 * GIB > free
                     or time.monotonic() - t0 > max_seconds):
@@ -87,24 +101,23 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
                 held.append(torch.empty(filler_bytes, dtype=torch.uint8, device=device))
             filled += step_bytes
             cand = zeros(bytes_b)
-            res = split_probe(handle, a, cand)
+            same, cross, full = summary(split_probe(handle, a, cand))
             report["tries"] += 1
             if log:
-                log(f"{filled / GIB:.0f} GiB of fillers: same {res[0]:.0f} GB/s, split {res[1]:.0f} GB/s")
-            if res[1] >= min_gain * res[0]:
-                chosen = cand
-                report.update(placed=True, filler_GiB=filled / GIB, same_GBps=res[0], cross_GBps=res[1])
+                log(f"{filled / GIB:.0f} GiB of fillers: same {same:.0f} GB/s, split {cross:.0f} GB/s")
+            if full or cross > report["cross_GBps"]:
+                held.append(best)
+                best = cand
+                report.update(placed=full, filler_GiB=filled / GIB, same_GBps=same, cross_GBps=cross)
             else:
                 held.append(cand)
             del cand
     except torch.cuda.OutOfMemoryError:
         pass
-    if chosen is not None:
-        b = chosen
     del held
     torch.cuda.empty_cache()
     report["seconds"] = time.monotonic() - t0
-    return a, b, report
+    return a, best, report
 
 
 def _device_map(block_gib: int = 2, reserve_gib: int = 6) -> None:
