@@ -10,7 +10,7 @@ import torch
 
 import oracle
 import ramtorch_amd
-from bench import HP, fill_tensor, llama3_8b_shapes, numel
+from bench import HP, fill_tensor, llama3_8b_shapes, numel, small_tensor_shapes
 from ramtorch_amd import _native as N
 from ramtorch_amd import functional as F
 
@@ -119,3 +119,90 @@ def test_philox_block_index_above_32_bits():
     for name, t, want in (("p", e.p, po), ("m", e.m, mo), ("v", e.v, vo)):
         assert int((bits16(t) != want).sum()) == 0, name
     h.close()
+
+
+def test_config2_every_tensor_matches_oracle():
+    """Config 2 at full size: 20 000 tensors of 1..4096 elements plus 64 of 1024 x 1024, one step
+    through AdamW.step (descriptors gathered in C++ when the helper is built), every tensor
+    compared bit for bit."""
+    dev = "cuda:0"
+    shapes = small_tensor_shapes()
+    assert len(shapes) == 20_064
+    params, grads, before = [], [], []
+    rng = np.random.default_rng(5)
+    for i, shp in enumerate(shapes):
+        n = numel(shp)
+        p, g, m, v = oracle.synth_inputs(n, int(rng.integers(0, 1 << 30)))
+        t = torch.from_numpy(p.view(np.int16).copy()).view(torch.bfloat16).view(shp).to(dev)
+        params.append(torch.nn.Parameter(t, requires_grad=False))
+        grads.append(torch.from_numpy(g.view(np.int16).copy()).view(torch.bfloat16).view(shp).to(dev))
+        before.append((p, g, m, v))
+    opt = ramtorch_amd.AdamW(params, storage_device="cuda", seed=1234, **HP)
+    for p, g, (_, _, m, v) in zip(params, grads, before):
+        p.grad = g
+        st = opt.state[p]
+        st["step"] = 99
+        st["ema"].copy_(torch.from_numpy(m.view(np.int16).copy()).view(torch.bfloat16).view(p.shape))
+        st["ema_squared"].copy_(torch.from_numpy(v.view(np.int16).copy()).view(torch.bfloat16).view(p.shape))
+    opt.step()
+    torch.cuda.synchronize()
+    sc = oracle.scalars_from_hparams(step=100, **HP)
+    bad = []
+    for i, (p, (p0, g0, m0, v0)) in enumerate(zip(params, before)):
+        po, mo, vo = p0.copy(), m0.copy(), v0.copy()
+        oracle.step_tensor(po, g0, mo, vo, sc, seed=1234, step=100, tensor_id=i)
+        st = opt.state[p]
+        if (st["step"] != 100 or (bits16(p) != po).any() or (bits16(st["ema"]) != mo).any()
+                or (bits16(st["ema_squared"]) != vo).any()):
+            bad.append(i)
+    assert not bad, f"{len(bad)} of {len(params)} tensors differ, first {bad[:5]}"
+
+
+def test_config4_layout_sampled_windows_match_oracle():
+    """Config 4 at full size: bf16 p / ema, fp32 gradients scaled by 1024, fp32 ema_squared, global-norm
+    clip to 1.0.  The norm is an order-dependent sum (checked to 1e-5 relative against float64 partial
+    sums on the GPU); given the coefficient the kernel used, sampled windows are bit-exact."""
+    dev = "cuda:0"
+    shapes = llama3_8b_shapes()
+    params, grads = [], []
+    for i, shp in enumerate(shapes):
+        params.append(torch.nn.Parameter(fill_tensor(shp, "p", 1234 + 4 * i, torch.bfloat16, dev), requires_grad=False))
+    for i, shp in enumerate(shapes):
+        grads.append(fill_tensor(shp, "g", 1234 + 4 * i + 1, torch.float32, dev).mul_(1024.0))
+    opt = ramtorch_amd.AdamW(params, storage_device="cuda", seed=1234, loss_scale=1024.0, max_grad_norm=1.0,
+                             ema_squared_dtype=torch.float32, **HP)
+    for i, p in enumerate(params):
+        st = opt.state[p]
+        st["step"] = 99
+        st["ema"].copy_(fill_tensor(p.shape, "m", 1234 + 4 * i + 2, torch.bfloat16, dev))
+        st["ema_squared"].copy_(fill_tensor(p.shape, "v", 1234 + 4 * i + 3, torch.float32, dev))
+    rng = np.random.default_rng(9)
+    W = 4096
+    sizes = np.array([numel(s) for s in shapes], dtype=np.float64)
+    wins = []
+    for ti in rng.choice(len(shapes), size=24, p=sizes / sizes.sum()):
+        n = numel(shapes[ti])
+        wins.append((int(ti), int(rng.integers(0, max(1, (n - W) // 8 + 1))) * 8, min(W, n)))
+    wins += [(0, 0, W), (len(shapes) - 1, numel(shapes[-1]) - W, W), (8, 0, 4096)]
+    before = []
+    for ti, lo, ln in wins:
+        p, st = params[ti], opt.state[params[ti]]
+        before.append((bits16(p.view(-1)[lo:lo + ln]), grads[ti].view(-1)[lo:lo + ln].cpu().numpy().copy(),
+                       bits16(st["ema"].view(-1)[lo:lo + ln]), st["ema_squared"].view(-1)[lo:lo + ln].cpu().numpy().copy()))
+    want_sq = sum(float((g.double() / 1024.0).square().sum()) for g in grads)
+    opt.step(grads=dict(zip(params, grads)))
+    torch.cuda.synchronize()
+    norm, coef, found_inf = (float(opt.last_grad_norm[0]), np.float32(opt.last_grad_norm[1].item()),
+                             int(opt.last_grad_norm.view(torch.int32)[2]))
+    assert found_inf == 0 and abs(norm - want_sq ** 0.5) <= 1e-5 * want_sq ** 0.5
+    assert coef == oracle.clip_coef(np.float32(norm), 1.0)
+    sc = oracle.scalars_from_hparams(step=100, inv_loss_scale=1.0 / 1024.0, apply_clip=True, **HP)
+    for (ti, lo, ln), (p0, g0, m0, v0) in zip(wins, before):
+        po, mo, vo = p0.copy(), m0.copy(), v0.copy()
+        oracle.step_tensor(po, g0, mo, vo, sc, g_dtype=oracle.DT_F32, v_dtype=oracle.DT_F32, clip_coef=coef, seed=1234,
+                           step=100, tensor_id=ti, elem_offset=lo)
+        st = opt.state[params[ti]]
+        assert int((bits16(params[ti].view(-1)[lo:lo + ln]) != po).sum()) == 0, (ti, lo)
+        assert int((bits16(st["ema"].view(-1)[lo:lo + ln]) != mo).sum()) == 0, (ti, lo)
+        got_v = st["ema_squared"].view(-1)[lo:lo + ln].cpu().numpy().view(np.uint32)
+        assert int((got_v != vo.view(np.uint32)).sum()) == 0, (ti, lo)
