@@ -206,3 +206,49 @@ def test_config4_layout_sampled_windows_match_oracle():
         assert int((bits16(st["ema"].view(-1)[lo:lo + ln]) != mo).sum()) == 0, (ti, lo)
         got_v = st["ema_squared"].view(-1)[lo:lo + ln].cpu().numpy().view(np.uint32)
         assert int((got_v != vo.view(np.uint32)).sum()) == 0, (ti, lo)
+
+
+def test_config3_streamed_set_sampled_windows_match_oracle():
+    """Config 3 at full size: parameters and both states of the 8 030 257 152-element set in pinned host
+    memory (48.2 GB), bf16 gradients on the GPU, 256 MB chunks.  One step through the three-stream
+    pipeline; sampled windows of the host arrays are bit-exact, including windows that straddle
+    chunk boundaries (a chunk holds 134 217 728 staged elements and cuts tensors at multiples of 8)."""
+    dev = "cuda:0"
+    shapes = llama3_8b_shapes()
+    params, grads = [], []
+    for i, shp in enumerate(shapes):
+        t = fill_tensor(shp, "p", 1234 + 4 * i, torch.bfloat16, dev).cpu().pin_memory()
+        params.append(torch.nn.Parameter(t, requires_grad=False))
+        grads.append(fill_tensor(shp, "g", 1234 + 4 * i + 1, torch.bfloat16, dev))
+    opt = ramtorch_amd.AdamW(params, storage_device="cpu", seed=1234, stream_chunk_bytes=256 << 20, **HP)
+    for i, p in enumerate(params):
+        st = opt.state[p]
+        st["step"] = 99
+        st["ema"].copy_(fill_tensor(p.shape, "m", 1234 + 4 * i + 2, torch.bfloat16, dev))
+        st["ema_squared"].copy_(fill_tensor(p.shape, "v", 1234 + 4 * i + 3, torch.bfloat16, dev))
+        assert st["ema"].is_pinned() and p.is_pinned()
+    rng = np.random.default_rng(13)
+    W = 4096
+    sizes = np.array([numel(s) for s in shapes], dtype=np.float64)
+    wins = []
+    for ti in rng.choice(len(shapes), size=30, p=sizes / sizes.sum()):
+        n = numel(shapes[ti])
+        wins.append((int(ti), int(rng.integers(0, max(1, (n - W) // 8 + 1))) * 8, min(W, n)))
+    chunk = (256 << 20) // 2
+    # the embedding (tensor 0, 525 336 576 elements) is cut at every multiple of `chunk`: windows across the cuts
+    wins += [(0, k * chunk - 2048, W) for k in (1, 2, 3)] + [(0, 0, W), (len(shapes) - 1, numel(shapes[-1]) - W, W)]
+    before = []
+    for ti, lo, ln in wins:
+        p, st = params[ti], opt.state[params[ti]]
+        # copies: for host tensors bits16() is a view of the live memory
+        before.append(tuple(bits16(t.view(-1)[lo:lo + ln]).copy() for t in (p, grads[ti], st["ema"], st["ema_squared"])))
+    opt.step(grads=dict(zip(params, grads)))   # returns when host memory is final
+    sc = oracle.scalars_from_hparams(step=100, **HP)
+    for (ti, lo, ln), (p0, g0, m0, v0) in zip(wins, before):
+        po, mo, vo = p0.copy(), m0.copy(), v0.copy()
+        oracle.step_tensor(po, g0, mo, vo, sc, seed=1234, step=100, tensor_id=ti, elem_offset=lo)
+        st = opt.state[params[ti]]
+        for name, t, want in (("p", params[ti], po), ("ema", st["ema"], mo), ("ema_squared", st["ema_squared"], vo)):
+            bad = int((bits16(t.view(-1)[lo:lo + ln]) != want).sum())
+            assert bad == 0, f"tensor {ti} window [{lo}, {lo + ln}) {name}: {bad} of {ln} values differ"
+    assert all(opt.state[p]["step"] == 100 for p in params)
