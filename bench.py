@@ -180,6 +180,7 @@ def main() -> int:
     ap.add_argument("--workload", default="llama8b", choices=["llama8b", "cfg0", "small", "mixed", "streamed", "hooked"])
     ap.add_argument("--layers", type=int, default=32, help="transformer layers of the Llama-shaped set")
     ap.add_argument("--stream-gb", type=float, default=48.2, help="upper bound on pinned host bytes (streamed)")
+    ap.add_argument("--stream-chunk-mb", type=int, default=256, help="bytes of bf16 per staged chunk and array (streamed)")
     ap.add_argument("--state-placement", default="auto", choices=["auto", "plain"],
                     help="AdamW(state_placement=...): 'auto' puts ema and ema_squared into different HBM regions")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -243,7 +244,7 @@ def main() -> int:
             params.append(torch.nn.Parameter(p, requires_grad=False))
             grads.append(fill_tensor(shp, "g", 1234 + 4 * i + 1, torch.bfloat16, dev))
         state_dtype = torch.bfloat16
-        opt_kw = dict(storage_device="cpu", seed=1234, stream_chunk_bytes=256 << 20)
+        opt_kw = dict(storage_device="cpu", seed=1234, stream_chunk_bytes=args.stream_chunk_mb << 20)
         bytes_per_elem = 12
         if wl == "hooked":
             gmap_needed = False
@@ -343,7 +344,7 @@ def main() -> int:
         stream_info = {"h2d_GBps": st["bytes_h2d"] / st["seconds"] / 1e9, "d2h_GBps": st["bytes_d2h"] / st["seconds"] / 1e9,
                        "seconds_last_call": st["seconds"], "host_bytes": 6 * total}
         # same-run pinned-copy peaks with the same chunk size
-        chunk = 256 << 20
+        chunk = args.stream_chunk_mb << 20
         hbuf = torch.empty(chunk, dtype=torch.uint8).pin_memory()
         dbuf = torch.empty(chunk, dtype=torch.uint8, device=dev)
         for name, (dst, src) in (("h2d", (dbuf, hbuf)), ("d2h", (hbuf, dbuf))):
