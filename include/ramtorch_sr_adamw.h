@@ -148,7 +148,9 @@ int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, cons
  * post-accumulate-grad hook that ramtorch/modules/linear.py:97-111 invokes
  * inside backward, instead of the D2H + H2D round trip of the gradient in
  * linear.py:416-427 / adamw.py:167).  Returns as soon as everything is
- * enqueued; *ticket (optional) identifies the call.  Until the ticket has
+ * enqueued (a call of more than 64 chunks is queued in batches of 64 and
+ * sleeps between them until the previous batch has left the pipeline);
+ * *ticket (optional) identifies the call.  Until the ticket has
  * completed the caller must keep every array of the call alive and must not
  * touch p / m / v.  Calls on one handle run in order and share the staging
  * buffers, so consecutive calls overlap like the chunks of one call.

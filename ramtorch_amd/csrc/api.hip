@@ -7,6 +7,7 @@
 #include <chrono>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <climits>
 #include <cstdint>
 #include <cstring>
@@ -95,6 +96,10 @@ struct Streamed {
     // into a word of pinned host memory; the host learns about completion by reading that word.
     uint64_t tickets_issued = 0;
     volatile uint64_t* ticket_word = nullptr;
+    // Progress: a second pinned word (ticket_word + 1) that receives the running chunk count at
+    // every batch boundary inside a long call; one call never has more than batch_chunks chunks
+    // queued on the streams (RT_STREAM_BATCH_CHUNKS in the environment overrides the default).
+    uint64_t batch_chunks = 64;
     bool ready = false;
     double bytes_h2d = 0, bytes_d2h = 0, seconds = 0;
     std::vector<hipEvent_t> tl_events;  // 4 per chunk when timing is on: H2D begin/end, D2H begin/end
@@ -684,8 +689,13 @@ static int streamed_init(rt_handle* h) {
     }
     void* word = nullptr;
     HIP_TRY(hipHostMalloc(&word, 64, hipHostMallocDefault));
-    *(volatile uint64_t*)word = 0;
+    ((volatile uint64_t*)word)[0] = 0;
+    ((volatile uint64_t*)word)[1] = 0;
     st.ticket_word = (volatile uint64_t*)word;
+    if (const char* e = getenv("RT_STREAM_BATCH_CHUNKS")) {
+        const long v = atol(e);
+        if (v > 0) st.batch_chunks = (uint64_t)v;
+    }
     st.ready = true;
     return RT_OK;
 }
@@ -750,18 +760,21 @@ static inline uint64_t tickets_done(const Streamed& st) {
     return st.ticket_word ? __atomic_load_n((const uint64_t*)st.ticket_word, __ATOMIC_ACQUIRE) : 0;
 }
 
+
 // Sleeps until ticket `want` has been published.  While the pipeline runs the host stays out
 // of the runtime: a thread spinning in a synchronise call, or polling events, was measured to
 // slow the copies down severalfold (the runtime resolves their cross-stream dependencies on
 // host threads).  The sleep is bounded: after kStallSeconds without a new ticket it returns
 // false and the caller falls back to a blocking synchronise, which also reports a failed device.
-static bool sleep_until_ticket(const Streamed& st, uint64_t want) {
+static bool sleep_until_word(const volatile uint64_t* word, uint64_t want) {
     constexpr double kStallSeconds = 60.0;
-    uint64_t seen = tickets_done(st);
+    if (!word) return false;
+    auto read_word = [word] { return __atomic_load_n((const uint64_t*)word, __ATOMIC_ACQUIRE); };
+    uint64_t seen = read_word();
     auto last_progress = std::chrono::steady_clock::now();
     while (seen < want) {
         std::this_thread::sleep_for(std::chrono::microseconds(100));
-        const uint64_t now_done = tickets_done(st);
+        const uint64_t now_done = read_word();
         const auto now = std::chrono::steady_clock::now();
         if (now_done != seen) {
             seen = now_done;
@@ -771,6 +784,10 @@ static bool sleep_until_ticket(const Streamed& st, uint64_t want) {
         }
     }
     return true;
+}
+
+static bool sleep_until_ticket(const Streamed& st, uint64_t want) {
+    return sleep_until_word(st.ticket_word, want);
 }
 
 static int streamed_wait(rt_handle* h) {
@@ -932,9 +949,21 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
             st.tl_events.push_back(e);
         }
     }
+    const uint64_t batch = st.batch_chunks;
     for (size_t c = 0; c < chunks.size(); ++c) {
         const int b = (int)((st.seq + c) & 1);
         const auto& segs = chunks[c];
+        // A long call is queued in batches, and the pipeline drains between them.  With a few
+        // hundred chunks waiting on the streams at once the copies of this pipeline were measured
+        // at well under half their rate, and queuing more while the streams are busy costs about
+        // as much; a drain costs one pipeline fill (about two chunk times) per batch.
+        if (c > 0 && c % batch == 0) {
+            hipLaunchKernelGGL(publish_ticket_kernel, dim3(1), dim3(1), 0, st.d2h,
+                               (uint64_t)(st.ticket_word + 1), st.seq + c);
+            HIP_TRY(hipGetLastError());
+            if (!sleep_until_word(st.ticket_word + 1, st.seq + c))
+                HIP_TRY(hipStreamSynchronize(st.d2h));  // stalled: block, and surface a device error
+        }
         // H2D: the buffer is free once the D2H of the chunk two back has finished
         if (st.used_buf[b]) HIP_TRY(hipStreamWaitEvent(st.h2d, st.d2h_done[b], 0));
         if (trace) HIP_TRY(hipEventRecord(st.tl_events[4 * c + 0], st.h2d));
