@@ -283,15 +283,17 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
     order.reserve(n);
     for (uint32_t i = 0; i < n; ++i)
         if (descs[i].numel != 0) order.push_back(i);
-    std::stable_sort(order.begin(), order.end(),
-                     [&](uint32_t a, uint32_t b) { return combo_of(descs[a]) < combo_of(descs[b]); });
+    const auto by_combo = [&](uint32_t a, uint32_t b) { return combo_of(descs[a]) < combo_of(descs[b]); };
+    if (!std::is_sorted(order.begin(), order.end(), by_combo))  // one combination is the common case
+        std::stable_sort(order.begin(), order.end(), by_combo);
 
     std::vector<DevTensor> tens(order.size());
     uint64_t total_chunks = 0;
+    auto it = set_of.end();
     for (size_t k = 0; k < order.size(); ++k) {
         const rt_tensor_desc& d = descs[order[k]];
         auto key = std::make_pair(d.scalars_idx, d.step);
-        auto it = set_of.find(key);
+        if (it == set_of.end() || it->first != key) it = set_of.find(key);  // neighbours mostly share a set
         if (it == set_of.end()) {
             DevScalars ds;
             memset(&ds, 0, sizeof(ds));
@@ -668,30 +670,34 @@ int rt_sr_copy(void* target_bf16, const float* source, uint64_t numel, const voi
 static int streamed_init(rt_handle* h) {
     Streamed& st = h->st;
     if (st.ready) return RT_OK;
-    HIP_TRY(hipStreamCreateWithFlags(&st.h2d, hipStreamNonBlocking));
-    HIP_TRY(hipStreamCreateWithFlags(&st.comp, hipStreamNonBlocking));
-    HIP_TRY(hipStreamCreateWithFlags(&st.d2h, hipStreamNonBlocking));
-    HIP_TRY(hipEventCreateWithFlags(&st.start, hipEventDisableTiming));
-    for (int b = 0; b < 2; ++b) {
-        HIP_TRY(hipEventCreateWithFlags(&st.h2d_done[b], hipEventDisableTiming));
-        HIP_TRY(hipEventCreateWithFlags(&st.comp_done[b], hipEventDisableTiming));
-        HIP_TRY(hipEventCreateWithFlags(&st.d2h_done[b], hipEventDisableTiming));
-    }
+    // Every step creates only what is still missing, so a call that failed halfway (out of
+    // memory, say) can be repeated without leaking what the first attempt created.
+    for (hipStream_t* s : {&st.h2d, &st.comp, &st.d2h})
+        if (!*s) HIP_TRY(hipStreamCreateWithFlags(s, hipStreamNonBlocking));
+    for (hipEvent_t* e : {&st.start, &st.h2d_done[0], &st.h2d_done[1], &st.comp_done[0], &st.comp_done[1],
+                          &st.d2h_done[0], &st.d2h_done[1]})
+        if (!*e) HIP_TRY(hipEventCreateWithFlags(e, hipEventDisableTiming));
     // Table memory for the calls in flight is set aside now: allocating (device or pinned
     // host memory) while the copy pipeline runs stalls the copies for tens of milliseconds.
-    st.ring.resize(kTablePool);
+    if (st.ring.size() < kTablePool) st.ring.resize(kTablePool);
     for (auto& r : st.ring) {
         int rc = dev_reserve(r.dev, kTablePoolBytes);
         if (rc != RT_OK) return rc;
+        if (r.host) continue;
         hipError_t e = hipHostMalloc(&r.host, kTablePoolBytes, hipHostMallocDefault);
-        if (e != hipSuccess) return fail(RT_ENOMEM, "hipHostMalloc(%zu) failed: %s", kTablePoolBytes, hipGetErrorString(e));
+        if (e != hipSuccess) {
+            r.host = nullptr;
+            return fail(RT_ENOMEM, "hipHostMalloc(%zu) failed: %s", kTablePoolBytes, hipGetErrorString(e));
+        }
         r.host_cap = kTablePoolBytes;
     }
-    void* word = nullptr;
-    HIP_TRY(hipHostMalloc(&word, 64, hipHostMallocDefault));
-    ((volatile uint64_t*)word)[0] = 0;
-    ((volatile uint64_t*)word)[1] = 0;
-    st.ticket_word = (volatile uint64_t*)word;
+    if (!st.ticket_word) {
+        void* word = nullptr;
+        HIP_TRY(hipHostMalloc(&word, 64, hipHostMallocDefault));
+        ((volatile uint64_t*)word)[0] = 0;
+        ((volatile uint64_t*)word)[1] = 0;
+        st.ticket_word = (volatile uint64_t*)word;
+    }
     if (const char* e = getenv("RT_STREAM_BATCH_CHUNKS")) {
         const long v = atol(e);
         if (v > 0) st.batch_chunks = (uint64_t)v;

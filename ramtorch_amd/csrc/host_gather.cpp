@@ -15,6 +15,7 @@
 #include <ATen/core/Tensor.h>
 
 #include <cstdint>
+#include <algorithm>
 #include <cstring>
 #include <vector>
 
@@ -69,6 +70,85 @@ inline bool dense_on(const at::Tensor& t, int dev) {
     return dev >= 0 ? (t.is_cuda() && t.get_device() == dev) : t.is_cpu();
 }
 
+// The walk below is a chain of dependent loads per tensor (list item -> Python wrapper ->
+// TensorImpl -> autograd meta -> gradient -> storage, and the same through the state dict), and
+// with tens of thousands of tensors none of it is in cache: the chain's latency is the cost.
+// Warm runs ahead of the main loop as a software pipeline: level k of the chain is prefetched
+// for tensor i + (kLevels - k) * kLead while tensor i is processed, so each level finds the
+// previous one already in cache.  It reads what the main loop reads and decides nothing.
+constexpr int kLevels = 5;
+constexpr Py_ssize_t kLead = 6;
+constexpr Py_ssize_t kRing = 64;  // > kLevels * kLead
+
+inline void touch(const void* p, int lines = 1) {
+    const char* c = static_cast<const char*>(p);
+    for (int k = 0; k < lines; ++k) __builtin_prefetch(c + 64 * k, 0, 3);
+}
+
+struct Warm {
+    PyObject* params;
+    PyObject* states;
+    Py_ssize_t n;
+    const c10::TensorImpl* impl[kRing][4];
+    PyObject* obj[kRing][3];
+
+    void level(int k, Py_ssize_t i) {
+        if (i < 0 || i >= n) return;
+        const Py_ssize_t r = i % kRing;
+        PyObject* po = PyList_GET_ITEM(params, i);
+        PyObject* so = PyList_GET_ITEM(states, i);
+        switch (k) {
+            case 0:  // wrappers and dict headers
+                touch(po);
+                touch(so);
+                break;
+            case 1:  // TensorImpl of the param; key table of the dict
+                impl[r][0] = exact_tensor(po) ? THPVariable_Unpack(po).unsafeGetTensorImpl() : nullptr;
+                if (impl[r][0]) touch(impl[r][0], 4);
+                if (PyDict_CheckExact(so)) touch(reinterpret_cast<PyDictObject*>(so)->ma_keys, 4);
+                break;
+            case 2:  // autograd meta + storage of the param; state objects
+                if (impl[r][0]) {
+                    touch(impl[r][0]->autograd_meta(), 2);
+                    touch(impl[r][0]->unsafe_storage().unsafeGetStorageImpl());
+                }
+                obj[r][0] = obj[r][1] = obj[r][2] = nullptr;
+                if (PyDict_CheckExact(so)) {
+                    obj[r][0] = PyDict_GetItem(so, k_ema);
+                    obj[r][1] = PyDict_GetItem(so, k_ema_squared);
+                    obj[r][2] = PyDict_GetItem(so, k_step);
+                    for (int j = 0; j < 3; ++j)
+                        if (obj[r][j]) touch(obj[r][j]);
+                }
+                break;
+            case 3:  // TensorImpl of the gradient and of both states
+                impl[r][1] = impl[r][2] = impl[r][3] = nullptr;
+                if (impl[r][0]) {
+                    const at::Tensor& g = THPVariable_Unpack(po).grad();
+                    if (g.defined()) impl[r][1] = g.unsafeGetTensorImpl();
+                }
+                for (int j = 0; j < 2; ++j)
+                    if (obj[r][j] && exact_tensor(obj[r][j]))
+                        impl[r][2 + j] = THPVariable_Unpack(obj[r][j]).unsafeGetTensorImpl();
+                for (int j = 1; j < 4; ++j)
+                    if (impl[r][j]) touch(impl[r][j], 4);
+                break;
+            default:  // their storages
+                for (int j = 1; j < 4; ++j)
+                    if (impl[r][j]) touch(impl[r][j]->unsafe_storage().unsafeGetStorageImpl());
+        }
+    }
+
+    // called before tensor i is processed
+    void ahead_of(Py_ssize_t i) {
+        if (i == 0) {  // fill the pipeline
+            for (int k = 0; k < kLevels; ++k)
+                for (Py_ssize_t j = 0; j < (kLevels - k) * kLead; ++j) level(k, j);
+        }
+        for (int k = 0; k < kLevels; ++k) level(k, i + (kLevels - k) * kLead);
+    }
+};
+
 // gather_group(params, states, dev, desc_addr, desc_cap, status_addr, scalars_base, tensor_id_base)
 //   -> (rows_written, [distinct new step values, in order of first use])
 // params: list of tensors; states: list of the per-param state dicts (same order);
@@ -100,7 +180,12 @@ PyObject* gather_group(PyObject*, PyObject* const* args, Py_ssize_t nargs) {
     }
     std::vector<long long> steps;
     Py_ssize_t w = 0;
+    Warm warm;
+    warm.params = params;
+    warm.states = states;
+    warm.n = n;
     for (Py_ssize_t i = 0; i < n; ++i) {
+        warm.ahead_of(i);
         status[i] = kPython;
         PyObject* po = PyList_GET_ITEM(params, i);
         PyObject* so = PyList_GET_ITEM(states, i);
