@@ -262,9 +262,9 @@ def main() -> int:
                                                 generator=torch.Generator(dev).manual_seed(1234 + k))
                                   for k in (1, 2, 3))}
     gmap = dict(zip(params, grads))
-    if wl == "small":
-        # bf16 gradients of bf16 params live in .grad, as after a backward pass; with this many
-        # tensors step() then collects its descriptors in C++
+    if wl in ("small", "llama8b"):
+        # bf16 gradients of bf16 params live in .grad, as after a backward pass; from 256
+        # tensors on step() then collects its descriptors in C++
         for p, g in zip(params, grads):
             p.grad = g
         gmap = None
