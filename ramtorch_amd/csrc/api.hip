@@ -167,24 +167,29 @@ static KernelPair pick_noise(int noise) {
         return {sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_PHILOX>, sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_PHILOX>};
     }
 }
-template <int P, int G, int M>
-static KernelPair pick_v(int v, int noise) {
-    return v == RT_DT_BF16 ? pick_noise<P, G, M, RT_DT_BF16>(noise) : pick_noise<P, G, M, RT_DT_F32>(noise);
-}
+// State dtype pairs the templated kernels are instantiated for: every bf16 / fp32 mix, and both fp16.
 template <int P, int G>
-static KernelPair pick_m(int m, int v, int noise) {
-    return m == RT_DT_BF16 ? pick_v<P, G, RT_DT_BF16>(v, noise) : pick_v<P, G, RT_DT_F32>(v, noise);
+static KernelPair pick_mv(int m, int v, int noise) {
+    if (m == RT_DT_F16) return pick_noise<P, G, RT_DT_F16, RT_DT_F16>(noise);
+    if (m == RT_DT_BF16)
+        return v == RT_DT_BF16 ? pick_noise<P, G, RT_DT_BF16, RT_DT_BF16>(noise)
+                               : pick_noise<P, G, RT_DT_BF16, RT_DT_F32>(noise);
+    return v == RT_DT_BF16 ? pick_noise<P, G, RT_DT_F32, RT_DT_BF16>(noise) : pick_noise<P, G, RT_DT_F32, RT_DT_F32>(noise);
 }
 template <int P>
 static KernelPair pick_g(int g, int m, int v, int noise) {
     switch (g) {
-        case RT_DT_BF16: return pick_m<P, RT_DT_BF16>(m, v, noise);
-        case RT_DT_F32: return pick_m<P, RT_DT_F32>(m, v, noise);
-        default: return pick_m<P, RT_DT_F16>(m, v, noise);
+        case RT_DT_BF16: return pick_mv<P, RT_DT_BF16>(m, v, noise);
+        case RT_DT_F32: return pick_mv<P, RT_DT_F32>(m, v, noise);
+        default: return pick_mv<P, RT_DT_F16>(m, v, noise);
     }
 }
 static KernelPair pick_kernel(int p, int g, int m, int v, int noise) {
-    return p == RT_DT_BF16 ? pick_g<RT_DT_BF16>(g, m, v, noise) : pick_g<RT_DT_F32>(g, m, v, noise);
+    switch (p) {
+        case RT_DT_BF16: return pick_g<RT_DT_BF16>(g, m, v, noise);
+        case RT_DT_F32: return pick_g<RT_DT_F32>(g, m, v, noise);
+        default: return pick_g<RT_DT_F16>(g, m, v, noise);
+    }
 }
 
 static inline uint32_t dtypes_of(const rt_tensor_desc& d) {
@@ -192,15 +197,17 @@ static inline uint32_t dtypes_of(const rt_tensor_desc& d) {
            ((uint32_t)d.v_dtype << 6);
 }
 
-// Tensors with an fp16 or fp64 param or state all go to the one runtime-typed kernel.
+// Tensors with an fp64 array, or with fp16 states in any other pairing than both fp16, all go to the
+// one runtime-typed kernel.
 constexpr uint32_t kComboAny = 0x100u;
 
-static inline bool compiled_pmv(int dt) { return dt == RT_DT_BF16 || dt == RT_DT_F32; }
+static inline bool compiled_combo(const rt_tensor_desc& d) {
+    if (d.p_dtype == RT_DT_F64 || d.m_dtype == RT_DT_F64 || d.v_dtype == RT_DT_F64) return false;
+    return (d.m_dtype == RT_DT_F16) == (d.v_dtype == RT_DT_F16);
+}
 
 // Launch group of a tensor: its dtype combination when the templated kernels cover it.
-static inline uint32_t combo_of(const rt_tensor_desc& d) {
-    return (compiled_pmv(d.p_dtype) && compiled_pmv(d.m_dtype) && compiled_pmv(d.v_dtype)) ? dtypes_of(d) : kComboAny;
-}
+static inline uint32_t combo_of(const rt_tensor_desc& d) { return compiled_combo(d) ? dtypes_of(d) : kComboAny; }
 
 // ---------------------------------------------------------------------------
 // argument validation shared by the resident and streamed entry points

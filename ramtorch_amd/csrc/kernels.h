@@ -161,12 +161,31 @@ __device__ __forceinline__ u32x4 sr_pack(const float (&x)[8], u32x4 noise) {
     return r;
 }
 
-// Write-back of one array: bf16 targets are stochastically rounded, fp32
-// targets are stored as they are.
+// fp32 -> IEEE half, round to nearest even (v_cvt_f16_f32: gradual underflow, overflow to infinity),
+// which is what a plain copy_ into an fp16 tensor does; two results per word.
+// The value converted must be the fp32 result as rounded: left to itself the compiler folds the
+// conversion into the fused multiply-add that produced it (v_fma_mixlo_f16: one rounding, straight
+// to fp16), which differs from round-to-fp32-then-to-fp16 in the last bit of ~0.5 % of the results.
+// The empty asm makes the fp32 value opaque at no cost.
+__device__ __forceinline__ uint32_t f16_bits(float x) {
+    asm volatile("" : "+v"(x));
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)x);
+}
+__device__ __forceinline__ uint32_t f16_pair(float lo, float hi) { return f16_bits(lo) | (f16_bits(hi) << 16); }
+__device__ __forceinline__ u32x4 f16_pack(const float (&x)[8]) {
+    u32x4 r;
+    r.x = f16_pair(x[0], x[1]); r.y = f16_pair(x[2], x[3]); r.z = f16_pair(x[4], x[5]); r.w = f16_pair(x[6], x[7]);
+    return r;
+}
+
+// Write-back of one array: bf16 targets are stochastically rounded, fp16 targets rounded to
+// nearest, fp32 targets stored as they are.
 template <int DT>
 __device__ __forceinline__ void store_out(uint64_t base, uint64_t i, const float (&x)[8], u32x4 noise) {
     if constexpr (DT == RT_DT_BF16) {
         stg128(base + i * 2, sr_pack(x, noise));
+    } else if constexpr (DT == RT_DT_F16) {
+        stg128(base + i * 2, f16_pack(x));
     } else {
         u32x4 a, b;
         a.x = f2u(x[0]); a.y = f2u(x[1]); a.z = f2u(x[2]); a.w = f2u(x[3]);
@@ -179,8 +198,8 @@ __device__ __forceinline__ void store_out(uint64_t base, uint64_t i, const float
 template <int DT>
 __device__ __forceinline__ void store_out_guarded(uint64_t base, uint64_t i, uint64_t n, const float (&x)[8],
                                                   u32x4 noise) {
-    if constexpr (DT == RT_DT_BF16) {
-        const u32x4 r = sr_pack(x, noise);
+    if constexpr (DT == RT_DT_BF16 || DT == RT_DT_F16) {
+        const u32x4 r = DT == RT_DT_BF16 ? sr_pack(x, noise) : f16_pack(x);
         const uint32_t w[4] = {r.x, r.y, r.z, r.w};
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
@@ -391,6 +410,11 @@ __device__ __forceinline__ void store_out4(uint64_t base, uint64_t e, const floa
         w.x = __builtin_amdgcn_perm(f2u(x[1]) + (noise.x >> 16), f2u(x[0]) + (noise.x & 0xFFFFu), 0x07060302u);
         w.y = __builtin_amdgcn_perm(f2u(x[3]) + (noise.y >> 16), f2u(x[2]) + (noise.y & 0xFFFFu), 0x07060302u);
         stg64(base + e * 2, w);
+    } else if constexpr (DT == RT_DT_F16) {
+        u32x2 w;
+        w.x = f16_pair(x[0], x[1]);
+        w.y = f16_pair(x[2], x[3]);
+        stg64(base + e * 2, w);
     } else {
         u32x4 a;
         a.x = f2u(x[0]); a.y = f2u(x[1]); a.z = f2u(x[2]); a.w = f2u(x[3]);
@@ -588,7 +612,9 @@ __global__ __launch_bounds__(kThreads) void sr_adamw_generic_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// Runtime-typed kernel: tensors whose param or states are kept in fp16 or fp64.
+// Runtime-typed kernel: tensors with an fp64 array, or with one fp16 state next
+// to a state of another dtype (the templated kernels cover fp16 params and a
+// pair of fp16 states).
 // The reference upcasts every dtype to fp32 (adamw.py:160-170) and writes
 // anything that is not bf16 back with a plain copy_ (adamw.py:208,214,221-222):
 // fp16 is rounded to nearest even (v_cvt_f16_f32), fp64 widened exactly; an
@@ -609,7 +635,7 @@ __device__ __forceinline__ float load_any(uint64_t base, uint32_t dt, uint64_t i
 __device__ __forceinline__ void store_any(uint64_t base, uint32_t dt, uint64_t idx, float x, uint32_t noise16) {
     switch (dt) {
         case RT_DT_BF16: stg16(base + idx * 2, (f2u(x) + noise16) >> 16); break;
-        case RT_DT_F16: stg16(base + idx * 2, __builtin_bit_cast(uint16_t, (_Float16)x)); break;
+        case RT_DT_F16: stg16(base + idx * 2, f16_bits(x)); break;
         case RT_DT_F64: *(RT_GLOBAL double*)(base + idx * 8) = (double)x; break;
         default: stg32f(base + idx * 4, x); break;
     }

@@ -213,9 +213,14 @@ def test_hyperparameters(handle, hp, step):
     (oracle.DT_F32, oracle.DT_BF16, oracle.DT_BF16, oracle.DT_BF16),
     (oracle.DT_BF16, oracle.DT_BF16, oracle.DT_F32, oracle.DT_BF16),
     # fp16 / fp64 params and states: upcast like everything else, plain copy_ on the way back
-    # (adamw.py:208,214,221-222) -- the runtime-typed kernel
+    # (adamw.py:208,214,221-222).  fp16 params, and states that are both fp16, have templated kernels ...
     (oracle.DT_F16, oracle.DT_F16, oracle.DT_F16, oracle.DT_F16),
     (oracle.DT_BF16, oracle.DT_BF16, oracle.DT_F16, oracle.DT_F16),
+    (oracle.DT_F16, oracle.DT_F16, oracle.DT_F32, oracle.DT_F32),
+    (oracle.DT_F16, oracle.DT_F32, oracle.DT_BF16, oracle.DT_BF16),
+    (oracle.DT_F32, oracle.DT_F16, oracle.DT_F16, oracle.DT_F16),
+    # ... fp64 anywhere, or one fp16 state next to another dtype, take the runtime-typed kernel
+    (oracle.DT_BF16, oracle.DT_BF16, oracle.DT_F16, oracle.DT_F32),
     (oracle.DT_F64, oracle.DT_F32, oracle.DT_BF16, oracle.DT_F64),
     (oracle.DT_F16, oracle.DT_BF16, oracle.DT_F64, oracle.DT_F32),
 ])
