@@ -772,21 +772,58 @@ template <int NOISE>
 __global__ __launch_bounds__(kThreads) void sr_copy_kernel(uint64_t target, uint64_t source, uint64_t n,
                                                            uint64_t noise, uint32_t seed_lo, uint32_t seed_hi,
                                                            int aligned) {
-    const uint64_t stride = (uint64_t)gridDim.x * kThreads * kVec;
-    for (uint64_t i = ((uint64_t)blockIdx.x * kThreads + threadIdx.x) * kVec; i < n; i += stride) {
-        const bool full = aligned && (i + kVec <= n);
-        const Raw8<RT_DT_F32> r = full ? load_raw<RT_DT_F32>(source, i) : load_raw_guarded<RT_DT_F32>(source, i, n);
-        float x[8];
-        decode<RT_DT_F32>(r, x);
-        u32x4 z;
-        if constexpr (NOISE == RT_NOISE_EXPLICIT) {
-            z = full ? ldg128(noise + i * 2) : load_raw_guarded<RT_DT_BF16>(noise, i, n).a;
+    // Whole blocks of 2048 elements of aligned arrays use the lane mapping of the wide update
+    // kernel (a lane owns 4 + 4 elements of its wave's 512-element block, so the fp32 loads are
+    // contiguous kilobytes across the wave) and the same neighbour swap of Philox halves; the last
+    // partial block and unaligned arrays go element by element under an index guard.
+    constexpr uint64_t kBlock = (uint64_t)kThreads * kVec;
+    constexpr uint32_t kHalf = 64 * kVec / 2;
+    const uint64_t n_blocks = (n + kBlock - 1) / kBlock;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const bool odd = (lane & 1u) != 0u;
+    for (uint64_t b = blockIdx.x; b < n_blocks; b += gridDim.x) {
+        const uint64_t base = b * kBlock;
+        if (aligned && base + kBlock <= n) {
+            const uint64_t blk = base + (uint64_t)wave * (64 * kVec);
+            u32x4 raw[2];
+            u32x2 z[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint64_t e = blk + (uint64_t)h * kHalf + lane * 4u;
+                raw[h] = ldg128(source + e * 4);
+                if constexpr (NOISE == RT_NOISE_EXPLICIT) z[h] = ldg64(noise + e * 2);
+            }
+            if constexpr (NOISE == RT_NOISE_PHILOX) {
+                const uint64_t first = (blk >> 3) + (lane >> 1);
+                const uint64_t mine = odd ? first + (kHalf >> 3) : first;
+                const u32x4 r = philox4x32_10((uint32_t)mine, (uint32_t)(mine >> 32), 3u, 0u, seed_lo, seed_hi);
+                const uint32_t g0 = swap_neighbour(odd ? r.x : r.z);
+                const uint32_t g1 = swap_neighbour(odd ? r.y : r.w);
+                z[0].x = odd ? g0 : r.x; z[0].y = odd ? g1 : r.y;
+                z[1].x = odd ? r.z : g0; z[1].y = odd ? r.w : g1;
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint64_t e = blk + (uint64_t)h * kHalf + lane * 4u;
+                float x[4];
+                decode4<RT_DT_F32>(raw[h], x);
+                store_out4<RT_DT_BF16>(target, e, x, z[h]);
+            }
         } else {
-            const uint64_t blk = i >> 3;
-            z = philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), 3u, 0u, seed_lo, seed_hi);
+            const uint64_t i = base + (uint64_t)threadIdx.x * kVec;
+            if (i >= n) continue;
+            const Raw8<RT_DT_F32> r = load_raw_guarded<RT_DT_F32>(source, i, n);
+            float x[8];
+            decode<RT_DT_F32>(r, x);
+            u32x4 z;
+            if constexpr (NOISE == RT_NOISE_EXPLICIT) {
+                z = load_raw_guarded<RT_DT_BF16>(noise, i, n).a;
+            } else {
+                const uint64_t blk = i >> 3;
+                z = philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), 3u, 0u, seed_lo, seed_hi);
+            }
+            store_out_guarded<RT_DT_BF16>(target, i, n, x, z);
         }
-        if (full) store_out<RT_DT_BF16>(target, i, x, z);
-        else store_out_guarded<RT_DT_BF16>(target, i, n, x, z);
     }
 }
 

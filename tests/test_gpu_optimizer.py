@@ -369,6 +369,18 @@ def test_copy_stochastic():
     cpu_tgt = torch.empty(n, dtype=torch.bfloat16)
     ramtorch_amd.copy_stochastic_(cpu_tgt, src, seed=42)
     assert nmis(cpu_tgt, tgt.cpu()) == 0
+    # whole 2048-element blocks, short tails, sizes below one block, unaligned views
+    big_t = torch.empty(3 * 2048 + 16, dtype=torch.bfloat16, device="cuda")
+    for off, m in ((0, 2048), (0, 3 * 2048), (0, 2047), (0, 7), (1, 2048 + 5), (3, 4096), (8, 3 * 2048)):
+        s_view, n_view, t_view = src[off:off + m], noise[off:off + m], big_t[off:off + m]
+        for kw in (dict(seed=9), dict(noise=n_view)):
+            big_t.zero_()
+            ramtorch_amd.copy_stochastic_(t_view, s_view, **kw)
+            torch.cuda.synchronize()
+            want = (oracle.sr_copy(s_view.cpu().numpy(), seed=9) if "seed" in kw
+                    else oracle.sr_copy(s_view.cpu().numpy(), noise=n_view.cpu().numpy()))
+            np.testing.assert_array_equal(bits16(t_view), want, err_msg=f"offset {off} n {m} {list(kw)}")
+            assert int(big_t[:off].view(torch.int16).abs().sum()) == 0 and int(big_t[off + m:].view(torch.int16).abs().sum()) == 0
     # the reference's own draw (adamw.py:10-21): a fresh generator seeded with `seed`
     src2 = src.view(-1)[:100_000].view(250, 400)
     tgt2 = torch.empty(250, 400, dtype=torch.bfloat16, device="cuda")
