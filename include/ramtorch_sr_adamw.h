@@ -202,12 +202,18 @@ int rt_sr_copy(void* target_bf16, const float* source, uint64_t numel, const voi
                uint64_t seed, void* stream);
 
 /*
- * Timing of the most recent rt_step_multi on this handle, measured with HIP
- * events recorded on the launch stream around the update kernels only.
- * Blocks until that work has finished.  Enabled by rt_set_timing(h, 1).
+ * Timing of rt_step_multi launches on this handle, measured with HIP events
+ * recorded on the launch stream around the update kernels only (a pair per
+ * launch, nothing is read or waited for while launches are being queued).
+ * Measurement only; nothing in the reference corresponds to it.
+ *   rt_set_timing(h, 1): start recording (and forget earlier launches); (h, 0): stop
+ *   rt_last_kernel_ms:   duration of the most recent timed launch; blocks until it has finished
+ *   rt_kernel_ms_history: durations of the min(cap, 256, launches since rt_set_timing) most
+ *                        recent timed launches, oldest first; blocks until they have finished
  */
 int rt_set_timing(rt_handle* h, int enabled);
 int rt_last_kernel_ms(rt_handle* h, float* ms);
+int rt_kernel_ms_history(rt_handle* h, float* out_ms, uint32_t cap, uint32_t* n_out);
 
 /*
  * Diagnostic, not in the reference: runs the memory traffic of the all-bf16

@@ -26,7 +26,7 @@ RT_HOST_P, RT_HOST_G, RT_HOST_M, RT_HOST_V = 1, 2, 4, 8
 #: every symbol the header declares
 EXPORTS = (
     "rt_version", "rt_last_error", "rt_create", "rt_destroy", "rt_step_multi", "rt_step_streamed",
-    "rt_grad_norm", "rt_row_means", "rt_sr_copy", "rt_set_timing", "rt_last_kernel_ms", "rt_streamed_stats",
+    "rt_grad_norm", "rt_row_means", "rt_sr_copy", "rt_set_timing", "rt_last_kernel_ms", "rt_kernel_ms_history", "rt_streamed_stats",
     "rt_stream_probe", "rt_streamed_timeline", "rt_streamed_plan",
     "rt_step_streamed_async", "rt_streamed_wait", "rt_streamed_completed",
 )
@@ -126,6 +126,8 @@ def lib() -> ctypes.CDLL:
     L.rt_set_timing.argtypes = [vp, i32]
     L.rt_last_kernel_ms.restype = i32
     L.rt_last_kernel_ms.argtypes = [vp, ctypes.POINTER(ctypes.c_float)]
+    L.rt_kernel_ms_history.restype = i32
+    L.rt_kernel_ms_history.argtypes = [vp, ctypes.POINTER(ctypes.c_float), u32, ctypes.POINTER(u32)]
     L.rt_stream_probe.restype = i32
     L.rt_stream_probe.argtypes = [vp, vp, vp, vp, vp, u64, i32, ctypes.POINTER(ctypes.c_float), vp]
     L.rt_streamed_timeline.restype = i32
@@ -231,6 +233,14 @@ class Handle:
         with self._lock:
             check(lib().rt_last_kernel_ms(self.ptr, ctypes.byref(ms)))
         return ms.value
+
+    def kernel_ms_history(self, cap: int = 256):
+        """Durations (ms) of the most recent timed launches since set_timing(True), oldest first."""
+        buf = (ctypes.c_float * cap)()
+        n = ctypes.c_uint32()
+        with self._lock:
+            check(lib().rt_kernel_ms_history(self.ptr, buf, cap, ctypes.byref(n)))
+        return [buf[i] for i in range(n.value)]
 
     def stream_probe(self, p, g, m, v, numel, reps=5, stream=0) -> float:
         """Mean ms per pass of the math-free traffic pattern (see rt_stream_probe)."""

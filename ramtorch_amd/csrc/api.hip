@@ -50,6 +50,7 @@ constexpr int kSlots = 2;            // table staging slots (host runs at most t
 constexpr size_t kTablePool = 8;     // table images of streamed calls in flight
 constexpr size_t kTablePoolBytes = 64 << 10;
 constexpr int kNormPartials = 2048;  // workgroups of the norm pass
+constexpr size_t kTimingRing = 256;   // timed launches whose durations can be read back
 constexpr uint64_t kMaxGrid = 0x7FFFFFFFull;  // workgroups of one launch (one per chunk of 8192 elements)
 
 struct DevBuf {
@@ -115,8 +116,11 @@ struct rt_handle {
     DevBuf norm_partials;
     std::vector<uint8_t> image;  // scratch for building a table image
     bool timing = false;
-    hipEvent_t t0 = nullptr, t1 = nullptr;
-    bool timed = false;
+    // Timing: a ring of event pairs, one pair per timed launch, so that the launches of a whole
+    // run can be timed without reading (and waiting for) any event in between.
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> tring;
+    uint64_t timed_launches = 0;  // since timing was last switched on
+    hipEvent_t t0 = nullptr, t1 = nullptr;  // rt_stream_probe's own pair
     Streamed st;
 };
 
@@ -446,12 +450,16 @@ static int launch_update(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, 
     TableSlot* slot = nullptr;
     int rc = stage_image(h, plan, stream, &slot);
     if (rc != RT_OK) return rc;
-    if (h->timing) HIP_TRY(hipEventRecord(h->t0, stream));
+    std::pair<hipEvent_t, hipEvent_t>* tp = nullptr;
+    if (h->timing) {
+        tp = &h->tring[h->timed_launches % kTimingRing];
+        HIP_TRY(hipEventRecord(tp->first, stream));
+    }
     rc = enqueue_kernels(plan, (const uint8_t*)slot->dev.ptr, seed, noise_mode, d_clip_coef, d_skip, stream);
     if (rc != RT_OK) return rc;
-    if (h->timing) {
-        HIP_TRY(hipEventRecord(h->t1, stream));
-        h->timed = true;
+    if (tp) {
+        HIP_TRY(hipEventRecord(tp->second, stream));
+        ++h->timed_launches;
     }
     HIP_TRY(hipEventRecord(slot->done, stream));
     slot->in_flight = true;
@@ -509,6 +517,10 @@ int rt_destroy(rt_handle* h) {
     if (h->norm_partials.ptr) (void)hipFree(h->norm_partials.ptr);
     if (h->t0) (void)hipEventDestroy(h->t0);
     if (h->t1) (void)hipEventDestroy(h->t1);
+    for (auto& pr : h->tring) {
+        if (pr.first) (void)hipEventDestroy(pr.first);
+        if (pr.second) (void)hipEventDestroy(pr.second);
+    }
     Streamed& st = h->st;
     for (int a = 0; a < 4; ++a)
         for (int b = 0; b < 2; ++b)
@@ -534,16 +546,44 @@ int rt_destroy(rt_handle* h) {
 
 int rt_set_timing(rt_handle* h, int enabled) {
     if (!h) return fail(RT_EINVAL, "handle is NULL");
+    if (enabled && h->tring.size() < kTimingRing) {
+        HIP_TRY(hipSetDevice(h->device));
+        h->tring.reserve(kTimingRing);
+        while (h->tring.size() < kTimingRing) {
+            std::pair<hipEvent_t, hipEvent_t> pr{nullptr, nullptr};
+            HIP_TRY(hipEventCreate(&pr.first));
+            hipError_t e = hipEventCreate(&pr.second);
+            if (e != hipSuccess) {
+                (void)hipEventDestroy(pr.first);
+                return fail(RT_EHIP, "hipEventCreate failed: %s (%d)", hipGetErrorString(e), (int)e);
+            }
+            h->tring.push_back(pr);
+        }
+    }
     h->timing = enabled != 0;
-    h->timed = false;
+    if (enabled) h->timed_launches = 0;
     return RT_OK;
 }
 
 int rt_last_kernel_ms(rt_handle* h, float* ms) {
     if (!h || !ms) return fail(RT_EINVAL, "NULL argument");
-    if (!h->timed) return fail(RT_EINVAL, "no timed launch on this handle (rt_set_timing first)");
-    HIP_TRY(hipEventSynchronize(h->t1));
-    HIP_TRY(hipEventElapsedTime(ms, h->t0, h->t1));
+    if (h->timed_launches == 0) return fail(RT_EINVAL, "no timed launch on this handle (rt_set_timing first)");
+    const auto& pr = h->tring[(h->timed_launches - 1) % kTimingRing];
+    HIP_TRY(hipEventSynchronize(pr.second));
+    HIP_TRY(hipEventElapsedTime(ms, pr.first, pr.second));
+    return RT_OK;
+}
+
+int rt_kernel_ms_history(rt_handle* h, float* out_ms, uint32_t cap, uint32_t* n_out) {
+    if (!h || !n_out || (cap > 0 && !out_ms)) return fail(RT_EINVAL, "NULL argument");
+    const uint64_t have = std::min<uint64_t>(h->timed_launches, kTimingRing);
+    const uint64_t n = std::min<uint64_t>(have, cap);
+    for (uint64_t k = 0; k < n; ++k) {  // oldest of the n most recent launches first
+        const auto& pr = h->tring[(h->timed_launches - n + k) % kTimingRing];
+        HIP_TRY(hipEventSynchronize(pr.second));
+        HIP_TRY(hipEventElapsedTime(&out_ms[k], pr.first, pr.second));
+    }
+    *n_out = (uint32_t)n;
     return RT_OK;
 }
 
@@ -1137,7 +1177,6 @@ int rt_stream_probe(rt_handle* h, void* p, const void* g, void* m, void* v, uint
     float ms = 0.0f;
     HIP_TRY(hipEventElapsedTime(&ms, h->t0, h->t1));
     *ms_out = ms / (float)reps;
-    h->timed = false;
     return RT_OK;
 }
 

@@ -374,6 +374,32 @@ def test_bad_arguments_are_rejected(handle):
         F.step_resident(handle, [e], [F.make_scalars(step=1, **HP0)], seed=0, explicit_noise=False)
 
 
+def test_kernel_timing_history(handle):
+    """rt_set_timing / rt_last_kernel_ms / rt_kernel_ms_history: one event pair per launch, read back
+    after the fact, oldest first; switching timing on again forgets earlier launches."""
+    n = 1 << 20
+    p, g, m, v = oracle.synth_inputs(n, 5)
+    e = F.Entry(p=dev16(p), g=dev16(g), m=dev16(m), v=dev16(v), step=1, scalars_idx=0, tensor_id=0)
+    sc = [F.make_scalars(step=1, **HP0)]
+    with pytest.raises(N.NativeError, match="no timed launch"):
+        handle.set_timing(True)
+        handle.last_kernel_ms()
+    for _ in range(5):
+        F.step_resident(handle, [e], sc, seed=1, explicit_noise=False)
+    hist = handle.kernel_ms_history()
+    assert len(hist) == 5 and all(0.0 < t < 50.0 for t in hist), hist
+    assert handle.kernel_ms_history(2) == hist[-2:]
+    assert handle.last_kernel_ms() == hist[-1]
+    handle.set_timing(True)
+    assert handle.kernel_ms_history() == []
+    F.step_resident(handle, [e], sc, seed=1, explicit_noise=False)
+    assert len(handle.kernel_ms_history()) == 1
+    handle.set_timing(False)
+    F.step_resident(handle, [e], sc, seed=1, explicit_noise=False)   # not recorded
+    assert len(handle.kernel_ms_history()) == 1
+    torch.cuda.synchronize()
+
+
 # ---- seeded random cases: sizes, dtypes, hyper-parameters, steps, noise modes, scaling -----------------
 def test_random_cases_match_the_oracle(handle):
     rng = np.random.default_rng(20240)
