@@ -357,3 +357,14 @@ def test_copies_and_unpickled_optimizers_keep_their_configuration():
     # load_state_dict goes through __setstate__ too and must leave the live configuration alone
     opt.load_state_dict(copy.deepcopy(opt.state_dict()))
     assert opt.max_inflight_calls == 5 and opt.loss_scale == 4.0
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asked for more it exits with a message instead of a number."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2", "--steps", "1", "--warmup", "0"],
+                         capture_output=True, text=True, timeout=120)
+    assert res.returncode != 0
+    assert "ONE GPU" in res.stderr and res.stdout.strip() == ""
