@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define RT_ABI_VERSION 1
+#define RT_ABI_VERSION 2
 
 /* error codes */
 #define RT_OK 0
@@ -137,10 +137,12 @@ int rt_step_multi(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const r
  * (grads ready) and returns after the last D2H has completed, so host memory
  * is final on return (the post-condition of the sync at adamw.py:232).
  * Results are bit-identical to rt_step_multi on the same data.
+ * d_clip_coef / d_skip: as for rt_step_multi (device pointers, may be NULL);
+ * they must be final for work queued on `stream` before the call.
  */
 int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
                      uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems,
-                     void* stream);
+                     const float* d_clip_coef, const uint32_t* d_skip, void* stream);
 
 /*
  * rt_step_streamed without the final wait, for callers that update one tensor
@@ -159,7 +161,7 @@ int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, cons
  */
 int rt_step_streamed_async(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
                            uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems,
-                           void* stream, uint64_t* ticket);
+                           const float* d_clip_coef, const uint32_t* d_skip, void* stream, uint64_t* ticket);
 int rt_streamed_wait(rt_handle* h);
 int rt_streamed_completed(rt_handle* h, uint64_t* ticket_done);
 
@@ -231,6 +233,26 @@ int rt_kernel_ms_history(rt_handle* h, float* out_ms, uint32_t cap, uint32_t* n_
  */
 int rt_stream_probe(rt_handle* h, void* p, const void* g, void* m, void* v, uint64_t numel, int reps,
                     float* ms_out, void* stream);
+
+/*
+ * Measurement only, nothing in the reference corresponds to it: what the host
+ * link gives plain pinned copies of `bytes` bytes, on the handle's own copy
+ * streams: out[0] = GB/s host to device, out[1] = GB/s device to host, each
+ * alone; out[2] = GB/s each way with both directions running at once (what the
+ * streamed pipeline does in steady state).  `reps` copies per figure after one
+ * warm-up copy.  Allocates and frees its own buffers; blocks until done.
+ */
+int rt_host_link_probe(rt_handle* h, uint64_t bytes, int reps, double out[3]);
+
+/*
+ * Self-test, nothing in the reference corresponds to it.  The update kernels
+ * take the square root of the second moment (adamw.py:193) with a shortened
+ * instruction sequence whenever a whole wavefront's values lie in
+ * [2^-96, +inf).  This runs that sequence and the compiler's correctly rounded
+ * sqrtf over every float of that range on the device and returns the number of
+ * bit patterns whose results differ (expected: 0).  Blocks until done.
+ */
+int rt_selftest_sqrt(rt_handle* h, uint64_t* mismatches);
 
 /*
  * Streamed-path statistics of the most recent rt_step_streamed:

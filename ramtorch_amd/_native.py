@@ -15,7 +15,7 @@ import weakref
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "_lib", "libramtorch_sr_adamw.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 RT_OK = 0
 RT_EINVAL, RT_EHIP, RT_ENOMEM, RT_EUNSUPPORTED = -1, -2, -3, -4
@@ -29,6 +29,7 @@ EXPORTS = (
     "rt_grad_norm", "rt_row_means", "rt_sr_copy", "rt_set_timing", "rt_last_kernel_ms", "rt_kernel_ms_history", "rt_streamed_stats",
     "rt_stream_probe", "rt_streamed_timeline", "rt_streamed_plan",
     "rt_step_streamed_async", "rt_streamed_wait", "rt_streamed_completed",
+    "rt_host_link_probe", "rt_selftest_sqrt",
 )
 
 
@@ -115,9 +116,13 @@ def lib() -> ctypes.CDLL:
     L.rt_step_multi.restype = i32
     L.rt_step_multi.argtypes = [vp, descs, u32, scal, u32, u64, i32, vp, vp, vp]
     L.rt_step_streamed.restype = i32
-    L.rt_step_streamed.argtypes = [vp, descs, u32, scal, u32, u64, i32, u64, vp]
+    L.rt_step_streamed.argtypes = [vp, descs, u32, scal, u32, u64, i32, u64, vp, vp, vp]
     L.rt_grad_norm.restype = i32
     L.rt_grad_norm.argtypes = [vp, descs, u32, ctypes.c_float, ctypes.c_float, vp, vp]
+    L.rt_host_link_probe.restype = i32
+    L.rt_host_link_probe.argtypes = [vp, u64, i32, ctypes.POINTER(ctypes.c_double)]
+    L.rt_selftest_sqrt.restype = i32
+    L.rt_selftest_sqrt.argtypes = [vp, ctypes.POINTER(u64)]
     L.rt_row_means.restype = i32
     L.rt_row_means.argtypes = [vp, vp, i32, u64, u64, ctypes.c_float, vp, vp]
     L.rt_sr_copy.restype = i32
@@ -133,7 +138,7 @@ def lib() -> ctypes.CDLL:
     L.rt_streamed_timeline.restype = i32
     L.rt_streamed_timeline.argtypes = [vp, ctypes.POINTER(ctypes.c_float), u32, ctypes.POINTER(u32)]
     L.rt_step_streamed_async.restype = i32
-    L.rt_step_streamed_async.argtypes = [vp, descs, u32, scal, u32, u64, i32, u64, vp, ctypes.POINTER(u64)]
+    L.rt_step_streamed_async.argtypes = [vp, descs, u32, scal, u32, u64, i32, u64, vp, vp, vp, ctypes.POINTER(u64)]
     L.rt_streamed_wait.restype = i32
     L.rt_streamed_wait.argtypes = [vp]
     L.rt_streamed_completed.restype = i32
@@ -193,17 +198,19 @@ class Handle:
             check(lib().rt_step_multi(self.ptr, descs, n, scalars, n_scalars, seed, noise_mode, d_clip_coef,
                                       d_skip, stream))
 
-    def step_streamed(self, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, stream=0):
+    def step_streamed(self, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, d_clip_coef=None,
+                      d_skip=None, stream=0):
         with self._lock:
             check(lib().rt_step_streamed(self.ptr, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems,
-                                         stream))
+                                         d_clip_coef, d_skip, stream))
 
-    def step_streamed_async(self, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, stream=0) -> int:
+    def step_streamed_async(self, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, d_clip_coef=None,
+                            d_skip=None, stream=0) -> int:
         """Enqueue only; returns the ticket of the call."""
         t = ctypes.c_uint64()
         with self._lock:
             check(lib().rt_step_streamed_async(self.ptr, descs, n, scalars, n_scalars, seed, noise_mode,
-                                               chunk_elems, stream, ctypes.byref(t)))
+                                               chunk_elems, d_clip_coef, d_skip, stream, ctypes.byref(t)))
         return t.value
 
     def streamed_wait(self) -> None:
@@ -219,6 +226,20 @@ class Handle:
     def grad_norm(self, descs, n, inv_loss_scale, max_norm, d_out, stream=0):
         with self._lock:
             check(lib().rt_grad_norm(self.ptr, descs, n, inv_loss_scale, max_norm, d_out, stream))
+
+    def host_link_probe(self, nbytes: int, reps: int = 8):
+        """Pinned-copy rates of the host link in GB/s: host to device, device to host, each way with both at once."""
+        out = (ctypes.c_double * 3)()
+        with self._lock:
+            check(lib().rt_host_link_probe(self.ptr, int(nbytes), int(reps), out))
+        return {"h2d_GBps": out[0], "d2h_GBps": out[1], "duplex_GBps_each_way": out[2]}
+
+    def selftest_sqrt(self) -> int:
+        """Number of floats in [2^-96, inf) on which the kernels' short sqrt differs from sqrtf (expected 0)."""
+        n = ctypes.c_uint64()
+        with self._lock:
+            check(lib().rt_selftest_sqrt(self.ptr, ctypes.byref(n)))
+        return n.value
 
     def row_means(self, g, g_dtype, rows, row_len, inv_loss_scale, d_row_mean, stream=0):
         with self._lock:

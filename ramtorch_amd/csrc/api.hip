@@ -115,6 +115,11 @@ struct rt_handle {
     uint64_t slot_counter = 0;
     DevBuf norm_partials;
     std::vector<uint8_t> image;  // scratch for building a table image
+    std::vector<DevTensor> tens;
+    std::vector<uint32_t> ranges;       // first unit of each tensor of the fast kernel
+    std::vector<DevTensor> fast_tens;   // their records
+    std::vector<PieceRef> pieces;
+    std::vector<ChunkRef> chunks;
     bool timing = false;
     // Timing: a ring of event pairs, one pair per timed launch, so that the launches of a whole
     // run can be timed without reading (and waiting for) any event in between.
@@ -146,12 +151,11 @@ static int dtype_size(int dt) { return dt == RT_DT_F32 ? 4 : dt == RT_DT_F64 ? 8
 // ---------------------------------------------------------------------------
 // kernel dispatch
 // ---------------------------------------------------------------------------
-using MultiKernel = void (*)(const DevTensor*, const ChunkRef*, const DevScalars*, uint32_t, uint32_t,
-                             const float*, const uint32_t*);
+using MultiKernel = void (*)(const LaunchArgs);
 
 struct KernelPair {
-    MultiKernel fast;     // chunks wholly inside an aligned tensor
-    MultiKernel generic;  // tails, unaligned tensors, debug outputs, centralization
+    MultiKernel fast;     // whole fast units of aligned tensors, plus (16-bit layouts, Philox) their pieces
+    MultiKernel generic;  // unaligned tensors, debug outputs, centralization, leftovers without a piece path
 };
 
 template <int P, int G, int M, int V>
@@ -268,25 +272,43 @@ namespace {
 
 struct Batch {            // tensors of one dtype combination inside a table image
     uint32_t combo;
-    uint32_t first_fast, n_fast;        // chunk range of the fast kernel
-    uint32_t first_generic, n_generic;  // chunk range of the generic kernel
+    uint32_t first_range, n_ranges, n_units;   // fast kernel: entries of the range list, fast units
+    uint32_t first_piece, n_pieces;            // pieces served by the fast kernel's first workgroups
+    uint32_t first_generic, n_generic;         // chunk range of the generic kernel
 };
 
 struct Plan {
-    size_t off_sets = 0, off_tensors = 0, off_chunks = 0, off_gdt = 0, bytes = 0;
+    size_t off_sets = 0, off_tensors = 0, off_ranges = 0, off_fast_tensors = 0, off_pieces = 0, off_chunks = 0,
+           off_gdt = 0, bytes = 0;
     uint32_t n_sets = 0, n_tensors = 0, n_chunks = 0;
+    DevScalars first_set;   // passed by value when n_sets == 1
     std::vector<Batch> batches;
 };
 
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+// All arrays 16 bit wide: the layouts whose fast kernel has a piece path.
+inline bool narrow_combo(uint32_t combo) {
+    if (combo & 0x100u) return false;
+    for (int k = 0; k < 4; ++k)
+        if (((combo >> (2 * k)) & 3u) == RT_DT_F32) return false;
+    return true;
+}
+
+enum class ImageFor { Update, Norm };
+
 }  // namespace
 
-// Lays out [DevScalars sets][DevTensor records][ChunkRef list][g dtype bytes]
-// in h->image.  Tensors are grouped by dtype combination so that each
-// combination is one contiguous chunk range = one launch.
+// Lays out [DevScalars sets][DevTensor records][first units][their DevTensor records][PieceRef pieces][ChunkRef list]
+// [g dtype bytes] in h->image.  Tensors are grouped by dtype combination so that each combination
+// is one contiguous range of every list = at most two launches.
+//   Update: whole fast units of plain tensors (16-byte aligned, no debug output, no centralization)
+//           become ranges; what such a tensor leaves over becomes pieces where the layout has a
+//           piece path (all arrays 16 bit, Philox noise), chunks of the generic kernel otherwise;
+//           every other tensor goes to the generic kernel chunk by chunk.
+//   Norm:   only the chunk list, over every element: whole chunks of aligned gradients first.
 static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
-                        bool want_explicit, Plan& plan) {
+                        bool want_explicit, ImageFor what, Plan& plan) {
     // (scalars_idx, step) -> set index
     std::map<std::pair<uint32_t, uint32_t>, uint32_t> set_of;
     std::vector<DevScalars> sets;
@@ -298,8 +320,8 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
     if (!std::is_sorted(order.begin(), order.end(), by_combo))  // one combination is the common case
         std::stable_sort(order.begin(), order.end(), by_combo);
 
-    std::vector<DevTensor> tens(order.size());
-    uint64_t total_chunks = 0;
+    std::vector<DevTensor>& tens = h->tens;
+    tens.resize(order.size());
     auto it = set_of.end();
     for (size_t k = 0; k < order.size(); ++k) {
         const rt_tensor_desc& d = descs[order[k]];
@@ -329,53 +351,113 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
         t.dtypes = dtypes_of(d);
         const uint64_t all = t.p | t.g | t.m | t.v | t.np | t.nm | t.nv;
         t.flags = (all & 15u) == 0 ? kFlagAligned : 0u;
-        total_chunks += (d.numel + kChunkElems - 1) / kChunkElems;
     }
 
-    plan.n_sets = (uint32_t)sets.size();
-    plan.n_tensors = (uint32_t)tens.size();
-    plan.n_chunks = (uint32_t)total_chunks;
-    plan.off_sets = 0;
-    plan.off_tensors = align_up(sets.size() * sizeof(DevScalars), 128);
-    plan.off_chunks = plan.off_tensors + align_up(tens.size() * sizeof(DevTensor), 128);
-    plan.off_gdt = plan.off_chunks + align_up(total_chunks * sizeof(ChunkRef), 128);
-    plan.bytes = plan.off_gdt + align_up(tens.size(), 128);
-    h->image.assign(plan.bytes, 0);
-    uint8_t* img = h->image.data();
-    if (!sets.empty()) memcpy(img + plan.off_sets, sets.data(), sets.size() * sizeof(DevScalars));
-    if (!tens.empty()) memcpy(img + plan.off_tensors, tens.data(), tens.size() * sizeof(DevTensor));
-    ChunkRef* cr = (ChunkRef*)(img + plan.off_chunks);
-    uint8_t* gdt = img + plan.off_gdt;
-    uint32_t c = 0;
+    // ---- work lists, combination by combination
+    std::vector<uint32_t>& ranges = h->ranges;
+    std::vector<DevTensor>& fast_tens = h->fast_tens;
+    std::vector<PieceRef>& pieces = h->pieces;
+    std::vector<ChunkRef>& chunks = h->chunks;
+    ranges.clear();
+    fast_tens.clear();
+    pieces.clear();
+    chunks.clear();
     plan.batches.clear();
-    // Per combination: first every chunk the fast kernel may take (whole chunks of
-    // aligned tensors without debug outputs or centralization), then the rest.
+    constexpr uint64_t unit = kFastUnitElems;
     size_t k0 = 0;
     while (k0 < order.size()) {
         const uint32_t combo = combo_of(descs[order[k0]]);
         size_t k1 = k0;
         while (k1 < order.size() && combo_of(descs[order[k1]]) == combo) ++k1;
-        Batch b{combo, c, 0, 0, 0};
-        auto n_whole = [&](size_t k) -> uint32_t {
-            const DevTensor& t = tens[k];
-            const bool plain = combo != kComboAny && (t.flags & kFlagAligned) && (t.dp | t.dm | t.dv | t.row_mean) == 0;
-            return plain ? (uint32_t)(t.numel / kChunkElems) : 0u;
+        Batch b{};
+        b.combo = combo;
+        b.first_range = (uint32_t)ranges.size();
+        b.first_piece = (uint32_t)pieces.size();
+        const bool has_pieces = what == ImageFor::Update && !want_explicit && narrow_combo(combo);
+        auto plain = [&](const DevTensor& t) {
+            return combo != kComboAny && (t.flags & kFlagAligned) && (t.dp | t.dm | t.dv | t.row_mean) == 0;
         };
-        for (size_t k = k0; k < k1; ++k) {
-            const uint32_t nw = n_whole(k);
-            for (uint32_t j = 0; j < nw; ++j) cr[c++] = ChunkRef{(uint32_t)k, j};
+        if (what == ImageFor::Norm) {
+            // the chunk list only: whole chunks of aligned gradients first, then the rest
+            b.first_generic = (uint32_t)chunks.size();
+            for (size_t k = k0; k < k1; ++k) {
+                const uint32_t nw = plain(tens[k]) ? (uint32_t)(tens[k].numel / kChunkElems) : 0u;
+                for (uint32_t j = 0; j < nw; ++j) chunks.push_back(ChunkRef{(uint32_t)k, j});
+            }
+            for (size_t k = k0; k < k1; ++k) {
+                const uint32_t nw = plain(tens[k]) ? (uint32_t)(tens[k].numel / kChunkElems) : 0u;
+                const uint32_t nc = (uint32_t)((tens[k].numel + kChunkElems - 1) / kChunkElems);
+                for (uint32_t j = nw; j < nc; ++j) chunks.push_back(ChunkRef{(uint32_t)k, j});
+            }
+            b.n_generic = (uint32_t)chunks.size() - b.first_generic;
+            plan.batches.push_back(b);
+            k0 = k1;
+            continue;
         }
-        b.n_fast = c - b.first_fast;
-        b.first_generic = c;
+        uint32_t units = 0;
         for (size_t k = k0; k < k1; ++k) {
-            const uint32_t nc = (uint32_t)((tens[k].numel + kChunkElems - 1) / kChunkElems);
-            for (uint32_t j = n_whole(k); j < nc; ++j) cr[c++] = ChunkRef{(uint32_t)k, j};
-            gdt[k] = descs[order[k]].g_dtype;
+            const DevTensor& t = tens[k];
+            if (!plain(t)) continue;
+            const uint32_t nu = (uint32_t)(t.numel / unit);
+            if (nu) {
+                ranges.push_back(units);
+                fast_tens.push_back(t);
+                units += nu;
+            }
+            if (has_pieces) {
+                for (uint64_t e = (uint64_t)nu * unit; e < t.numel; e += kPieceElems) {
+                    PieceRef r;
+                    memset(&r, 0, sizeof(r));
+                    const int ep = dtype_size(t.dtypes & 3u), eg = dtype_size((t.dtypes >> 2) & 3u),
+                              em = dtype_size((t.dtypes >> 4) & 3u), ev = dtype_size((t.dtypes >> 6) & 3u);
+                    r.p = t.p + e * ep; r.g = t.g + e * eg; r.m = t.m + e * em; r.v = t.v + e * ev;
+                    r.block = t.block_base + (e >> 3);
+                    r.count = (uint32_t)std::min<uint64_t>(kPieceElems, t.numel - e);
+                    r.tensor_id4 = t.tensor_id4;
+                    r.set_idx = t.set_idx;
+                    pieces.push_back(r);
+                }
+            }
         }
-        b.n_generic = c - b.first_generic;
+        b.n_ranges = (uint32_t)ranges.size() - b.first_range;
+        b.n_units = units;
+        b.n_pieces = (uint32_t)pieces.size() - b.first_piece;
+        b.first_generic = (uint32_t)chunks.size();
+        for (size_t k = k0; k < k1; ++k) {
+            const DevTensor& t = tens[k];
+            const uint32_t nc = (uint32_t)((t.numel + kChunkElems - 1) / kChunkElems);
+            uint32_t j0 = 0;
+            if (plain(t)) j0 = has_pieces ? nc : (uint32_t)(t.numel / kChunkElems);
+            for (uint32_t j = j0; j < nc; ++j) chunks.push_back(ChunkRef{(uint32_t)k, j});
+        }
+        b.n_generic = (uint32_t)chunks.size() - b.first_generic;
         plan.batches.push_back(b);
         k0 = k1;
     }
+
+    plan.n_sets = (uint32_t)sets.size();
+    plan.n_tensors = (uint32_t)tens.size();
+    plan.n_chunks = (uint32_t)chunks.size();
+    if (!sets.empty()) plan.first_set = sets[0];
+    plan.off_sets = 0;
+    plan.off_tensors = align_up(sets.size() * sizeof(DevScalars), 256);
+    plan.off_ranges = plan.off_tensors + align_up(tens.size() * sizeof(DevTensor), 128);
+    plan.off_fast_tensors = plan.off_ranges + align_up(ranges.size() * sizeof(uint32_t), 128);
+    plan.off_pieces = plan.off_fast_tensors + align_up(fast_tens.size() * sizeof(DevTensor), 128);
+    plan.off_chunks = plan.off_pieces + align_up(pieces.size() * sizeof(PieceRef), 128);
+    plan.off_gdt = plan.off_chunks + align_up(chunks.size() * sizeof(ChunkRef), 128);
+    plan.bytes = plan.off_gdt + (what == ImageFor::Norm ? align_up(tens.size(), 128) : 0);
+    h->image.assign(plan.bytes, 0);
+    uint8_t* img = h->image.data();
+    if (!sets.empty()) memcpy(img + plan.off_sets, sets.data(), sets.size() * sizeof(DevScalars));
+    if (!tens.empty()) memcpy(img + plan.off_tensors, tens.data(), tens.size() * sizeof(DevTensor));
+    if (!ranges.empty()) memcpy(img + plan.off_ranges, ranges.data(), ranges.size() * sizeof(uint32_t));
+    if (!fast_tens.empty())
+        memcpy(img + plan.off_fast_tensors, fast_tens.data(), fast_tens.size() * sizeof(DevTensor));
+    if (!pieces.empty()) memcpy(img + plan.off_pieces, pieces.data(), pieces.size() * sizeof(PieceRef));
+    if (!chunks.empty()) memcpy(img + plan.off_chunks, chunks.data(), chunks.size() * sizeof(ChunkRef));
+    if (what == ImageFor::Norm)
+        for (size_t k = 0; k < order.size(); ++k) img[plan.off_gdt + k] = descs[order[k]].g_dtype;
 }
 
 // Puts h->image into a free table slot (skipping the copy when the slot's
@@ -401,12 +483,21 @@ static int stage_image(rt_handle* h, const Plan& plan, hipStream_t stream, Table
         int rc = dev_reserve(s.dev, plan.bytes);
         if (rc != RT_OK) return rc;
     }
-    const bool same = s.valid_bytes == plan.bytes && memcmp(s.host, h->image.data(), plan.bytes) == 0;
-    if (!same && plan.bytes > 0) {
-        memcpy(s.host, h->image.data(), plan.bytes);
-        HIP_TRY(hipMemcpyAsync(s.dev.ptr, s.host, plan.bytes, hipMemcpyHostToDevice, stream));
-        s.valid_bytes = plan.bytes;
+    // Two regions: the DevScalars sets change with every step, the lists behind them only when the
+    // tensors do; each region is copied only if the device copy differs.
+    const size_t split = std::min(plan.off_tensors, plan.bytes);
+    const uint8_t* img = h->image.data();
+    const bool known = s.valid_bytes == plan.bytes;
+    if (split > 0 && !(known && memcmp(s.host, img, split) == 0)) {
+        memcpy(s.host, img, split);
+        HIP_TRY(hipMemcpyAsync(s.dev.ptr, s.host, split, hipMemcpyHostToDevice, stream));
     }
+    if (plan.bytes > split && !(known && memcmp((uint8_t*)s.host + split, img + split, plan.bytes - split) == 0)) {
+        memcpy((uint8_t*)s.host + split, img + split, plan.bytes - split);
+        HIP_TRY(hipMemcpyAsync((uint8_t*)s.dev.ptr + split, (uint8_t*)s.host + split, plan.bytes - split,
+                               hipMemcpyHostToDevice, stream));
+    }
+    s.valid_bytes = plan.bytes;
     *out = &s;
     return RT_OK;
 }
@@ -414,27 +505,43 @@ static int stage_image(rt_handle* h, const Plan& plan, hipStream_t stream, Table
 // Enqueues the update kernels of one table image that already sits in device memory at `base`.
 static int enqueue_kernels(const Plan& plan, const uint8_t* base, uint64_t seed, int noise_mode,
                            const float* d_clip_coef, const uint32_t* d_skip, hipStream_t stream) {
-    const DevScalars* sets = (const DevScalars*)(base + plan.off_sets);
-    const DevTensor* tens = (const DevTensor*)(base + plan.off_tensors);
-    const ChunkRef* chunks = (const ChunkRef*)(base + plan.off_chunks);
+    LaunchArgs a;
+    memset(&a, 0, sizeof(a));
+    a.tensors = (const DevTensor*)(base + plan.off_tensors);
+    a.sets = (const DevScalars*)(base + plan.off_sets);
+    a.clip_coef = d_clip_coef;
+    a.skip = d_skip;
+    a.seed_lo = (uint32_t)seed;
+    a.seed_hi = (uint32_t)(seed >> 32);
+    a.use_ks = plan.n_sets == 1 ? 1u : 0u;
+    a.ks = plan.first_set;
     for (const Batch& b : plan.batches) {
         KernelPair k;
         if (b.combo == kComboAny) {
-            k.fast = nullptr;  // n_fast is 0 for this group
+            k.fast = nullptr;  // no ranges and no pieces for this group
             k.generic = noise_mode == RT_NOISE_EXPLICIT ? sr_adamw_any_kernel<RT_NOISE_EXPLICIT>
                                                         : sr_adamw_any_kernel<RT_NOISE_PHILOX>;
         } else {
             k = pick_kernel(b.combo & 3, (b.combo >> 2) & 3, (b.combo >> 4) & 3, (b.combo >> 6) & 3, noise_mode);
         }
-        if (b.n_fast) {
-            hipLaunchKernelGGL(k.fast, dim3(b.n_fast), dim3(kThreads), 0, stream, tens, chunks + b.first_fast, sets,
-                               (uint32_t)seed, (uint32_t)(seed >> 32), d_clip_coef, d_skip);
+        a.first = (const uint32_t*)(base + plan.off_ranges) + b.first_range;
+        a.fast_tensors = (const DevTensor*)(base + plan.off_fast_tensors) + b.first_range;
+        a.n_ranges = b.n_ranges;
+        a.pieces = (const PieceRef*)(base + plan.off_pieces) + b.first_piece;
+        a.n_pieces = b.n_pieces;
+        a.n_piece_wgs = (b.n_pieces + 3u) / 4u;
+        a.chunks = (const ChunkRef*)(base + plan.off_chunks) + b.first_generic;
+        const uint64_t grid = (uint64_t)a.n_piece_wgs + b.n_units;
+        a.piece_rate = 0;  // only pieces, or none
+        if (a.n_piece_wgs != 0 && b.n_units != 0)
+            a.piece_rate = (uint32_t)((((uint64_t)a.n_piece_wgs << 32) + grid - 1) / grid);  // < 2^32: n_piece_wgs < grid
+        if (grid > kMaxGrid || b.n_generic > kMaxGrid) return fail(RT_EUNSUPPORTED, "too many workgroups in one launch");
+        if (grid) {
+            hipLaunchKernelGGL(k.fast, dim3((uint32_t)grid), dim3(kThreads), 0, stream, a);
             HIP_TRY(hipGetLastError());
         }
         if (b.n_generic) {
-            hipLaunchKernelGGL(k.generic, dim3(b.n_generic), dim3(kThreads), 0, stream, tens,
-                               chunks + b.first_generic, sets, (uint32_t)seed, (uint32_t)(seed >> 32), d_clip_coef,
-                               d_skip);
+            hipLaunchKernelGGL(k.generic, dim3(b.n_generic), dim3(kThreads), 0, stream, a);
             HIP_TRY(hipGetLastError());
         }
     }
@@ -445,8 +552,8 @@ static int launch_update(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, 
                          uint64_t seed, int noise_mode, const float* d_clip_coef, const uint32_t* d_skip,
                          hipStream_t stream) {
     Plan plan;
-    build_image(h, descs, n, scalars, noise_mode == RT_NOISE_EXPLICIT, plan);
-    if (plan.n_chunks == 0) return RT_OK;
+    build_image(h, descs, n, scalars, noise_mode == RT_NOISE_EXPLICIT, ImageFor::Update, plan);
+    if (plan.n_tensors == 0) return RT_OK;
     TableSlot* slot = nullptr;
     int rc = stage_image(h, plan, stream, &slot);
     if (rc != RT_OK) return rc;
@@ -632,7 +739,7 @@ int rt_grad_norm(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, float in
         d.p_dtype = d.g_dtype = d.m_dtype = d.v_dtype = RT_DT_BF16;
     }
     Plan plan;
-    build_image(h, gd.data(), n, &one, false, plan);
+    build_image(h, gd.data(), n, &one, false, ImageFor::Norm, plan);
     {
         // build_image keeps the input order inside one combination
         uint8_t* gdt = h->image.data() + plan.off_gdt;
@@ -861,8 +968,9 @@ static int streamed_wait(rt_handle* h) {
 
 // Validates and enqueues the whole pipeline of one call; does not wait for it.
 static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
-                            uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems, void* stream_,
-                            bool trace, uint64_t* ticket_out) {
+                            uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems,
+                            const float* d_clip_coef, const uint32_t* d_skip, void* stream_, bool trace,
+                            uint64_t* ticket_out) {
     if (!h) return fail(RT_EINVAL, "handle is NULL");
     int rc = validate(descs, n, scalars, n_scalars, noise_mode, /*allow_host=*/true);
     if (rc != RT_OK) return rc;
@@ -943,7 +1051,7 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
             pieces[c].push_back(q);
         }
         build_image(h, pieces[c].data(), (uint32_t)pieces[c].size(), scalars, noise_mode == RT_NOISE_EXPLICIT,
-                    plans[c]);
+                    ImageFor::Update, plans[c]);
         plan_off[c] = align_up(blob.size(), 256);
         blob.resize(plan_off[c] + plans[c].bytes);
         if (plans[c].bytes) memcpy(blob.data() + plan_off[c], h->image.data(), plans[c].bytes);
@@ -1042,8 +1150,8 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
 
         // compute
         HIP_TRY(hipStreamWaitEvent(st.comp, st.h2d_done[b], 0));
-        rc = enqueue_kernels(plans[c], (const uint8_t*)tab.dev.ptr + plan_off[c], seed, noise_mode, nullptr,
-                             nullptr, st.comp);
+        rc = enqueue_kernels(plans[c], (const uint8_t*)tab.dev.ptr + plan_off[c], seed, noise_mode, d_clip_coef,
+                             d_skip, st.comp);
         if (rc != RT_OK) return rc;
         HIP_TRY(hipEventRecord(st.comp_done[b], st.comp));
 
@@ -1087,10 +1195,11 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
 // what the streams hold.  Drain the streams and start over from a clean state; the error of the
 // failed call is what the caller sees.
 static int streamed_enqueue(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
-                            uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems, void* stream_,
-                            bool trace, uint64_t* ticket_out) {
-    const int rc = streamed_enqueue_impl(h, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, stream_,
-                                         trace, ticket_out);
+                            uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems,
+                            const float* d_clip_coef, const uint32_t* d_skip, void* stream_, bool trace,
+                            uint64_t* ticket_out) {
+    const int rc = streamed_enqueue_impl(h, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, d_clip_coef,
+                                         d_skip, stream_, trace, ticket_out);
     if (rc != RT_OK && h && h->st.ready) {
         char saved[sizeof(g_err)];
         memcpy(saved, g_err, sizeof(saved));
@@ -1107,11 +1216,13 @@ static int streamed_enqueue(rt_handle* h, const rt_tensor_desc* descs, uint32_t 
 }
 
 int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
-                     uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems, void* stream) {
+                     uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems,
+                     const float* d_clip_coef, const uint32_t* d_skip, void* stream) {
     if (!h) return fail(RT_EINVAL, "handle is NULL");
     const auto wall0 = std::chrono::steady_clock::now();
     const bool trace = h->timing;
-    int rc = streamed_enqueue(h, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, stream, trace, nullptr);
+    int rc = streamed_enqueue(h, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, d_clip_coef, d_skip,
+                              stream, trace, nullptr);
     if (rc != RT_OK) return rc;
     // Host memory is final on return; device-resident arrays are final for the caller's stream.
     rc = streamed_wait(h);
@@ -1125,10 +1236,11 @@ int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, cons
 }
 
 int rt_step_streamed_async(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
-                           uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems, void* stream,
-                           uint64_t* ticket) {
+                           uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems,
+                           const float* d_clip_coef, const uint32_t* d_skip, void* stream, uint64_t* ticket) {
     if (!h) return fail(RT_EINVAL, "handle is NULL");
-    return streamed_enqueue(h, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, stream, false, ticket);
+    return streamed_enqueue(h, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, d_clip_coef, d_skip,
+                            stream, false, ticket);
 }
 
 int rt_streamed_wait(rt_handle* h) {
@@ -1177,6 +1289,77 @@ int rt_stream_probe(rt_handle* h, void* p, const void* g, void* m, void* v, uint
     float ms = 0.0f;
     HIP_TRY(hipEventElapsedTime(&ms, h->t0, h->t1));
     *ms_out = ms / (float)reps;
+    return RT_OK;
+}
+
+int rt_host_link_probe(rt_handle* h, uint64_t bytes, int reps, double out[3]) {
+    if (!h || !out) return fail(RT_EINVAL, "NULL argument");
+    if (bytes == 0 || reps < 1) return fail(RT_EINVAL, "bytes and reps must be positive");
+    HIP_TRY(hipSetDevice(h->device));
+    int rc = streamed_init(h);
+    if (rc != RT_OK) return rc;
+    rc = streamed_wait(h);
+    if (rc != RT_OK) return rc;
+    Streamed& st = h->st;
+    void *hbuf[2] = {nullptr, nullptr}, *dbuf[2] = {nullptr, nullptr};
+    hipError_t e = hipSuccess;
+    for (int k = 0; k < 2 && e == hipSuccess; ++k) {
+        e = hipHostMalloc(&hbuf[k], bytes, hipHostMallocDefault);
+        if (e == hipSuccess) e = hipMalloc(&dbuf[k], bytes);
+    }
+    auto release = [&] {
+        for (int k = 0; k < 2; ++k) {
+            if (hbuf[k]) (void)hipHostFree(hbuf[k]);
+            if (dbuf[k]) (void)hipFree(dbuf[k]);
+        }
+    };
+    if (e != hipSuccess) {
+        release();
+        (void)hipGetLastError();
+        return fail(RT_ENOMEM, "allocating the probe buffers (%llu bytes each) failed: %s", (unsigned long long)bytes,
+                    hipGetErrorString(e));
+    }
+    memset(hbuf[0], 0, bytes);
+    memset(hbuf[1], 0, bytes);
+    using clock = std::chrono::steady_clock;
+    auto run = [&](bool up, bool down) -> double {   // seconds for `reps` copies each way
+        if (up) (void)hipMemcpyAsync(dbuf[0], hbuf[0], bytes, hipMemcpyHostToDevice, st.h2d);    // warm-up
+        if (down) (void)hipMemcpyAsync(hbuf[1], dbuf[1], bytes, hipMemcpyDeviceToHost, st.d2h);
+        (void)hipStreamSynchronize(st.h2d);
+        (void)hipStreamSynchronize(st.d2h);
+        const auto t0 = clock::now();
+        for (int r = 0; r < reps; ++r) {
+            if (up) (void)hipMemcpyAsync(dbuf[0], hbuf[0], bytes, hipMemcpyHostToDevice, st.h2d);
+            if (down) (void)hipMemcpyAsync(hbuf[1], dbuf[1], bytes, hipMemcpyDeviceToHost, st.d2h);
+        }
+        (void)hipStreamSynchronize(st.h2d);
+        (void)hipStreamSynchronize(st.d2h);
+        return std::chrono::duration<double>(clock::now() - t0).count();
+    };
+    const double total = (double)bytes * reps / 1e9;
+    out[0] = total / run(true, false);
+    out[1] = total / run(false, true);
+    out[2] = total / run(true, true);
+    release();
+    HIP_TRY(hipGetLastError());
+    return RT_OK;
+}
+
+int rt_selftest_sqrt(rt_handle* h, uint64_t* mismatches) {
+    if (!h || !mismatches) return fail(RT_EINVAL, "NULL argument");
+    HIP_TRY(hipSetDevice(h->device));
+    unsigned long long* d = nullptr;
+    HIP_TRY(hipMalloc((void**)&d, sizeof(*d)));
+    hipError_t e = hipMemset(d, 0, sizeof(*d));
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(sqrt_selftest_kernel, dim3(16384), dim3(kThreads), 0, nullptr, d);
+        e = hipGetLastError();
+    }
+    unsigned long long host = 0;
+    if (e == hipSuccess) e = hipMemcpy(&host, d, sizeof(host), hipMemcpyDeviceToHost);
+    (void)hipFree(d);
+    if (e != hipSuccess) return fail(RT_EHIP, "sqrt self-test failed: %s (%d)", hipGetErrorString(e), (int)e);
+    *mismatches = host;
     return RT_OK;
 }
 

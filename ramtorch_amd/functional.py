@@ -176,7 +176,8 @@ def step_resident(handle: N.Handle, entries: Sequence[Entry], scalars: Sequence[
 
 def step_streamed(handle: N.Handle, entries: Sequence[Entry], scalars: Sequence[N.RtScalars], *, seed: int,
                   explicit_noise: bool, chunk_elems: int, stream: Optional[int] = None,
-                  wait: bool = True) -> Optional[int]:
+                  wait: bool = True, clip_coef: Optional[torch.Tensor] = None,
+                  skip: Optional[torch.Tensor] = None, descs: Optional[np.ndarray] = None) -> Optional[int]:
     """Chunked H2D / update / D2H for tensors with CPU-resident arrays.  With
     ``wait`` (default) host memory is final when this returns.  Without it the
     call only enqueues and returns a ticket: until ``handle.streamed_completed()``
@@ -184,11 +185,12 @@ def step_streamed(handle: N.Handle, entries: Sequence[Entry], scalars: Sequence[
     tensors alive and leave p / m / v alone."""
     if not entries:
         return None
-    d = pack_descs(entries, streamed=True)
+    d = pack_descs(entries, streamed=True) if descs is None else descs
     if stream is None:
         stream = torch.cuda.current_stream(handle.device).cuda_stream
     args = (_descs_ptr(d), len(entries), scalars_array(scalars), len(scalars), seed & (2 ** 64 - 1),
-            N.RT_NOISE_EXPLICIT if explicit_noise else N.RT_NOISE_PHILOX, int(chunk_elems), stream)
+            N.RT_NOISE_EXPLICIT if explicit_noise else N.RT_NOISE_PHILOX, int(chunk_elems),
+            None if clip_coef is None else clip_coef.data_ptr(), None if skip is None else skip.data_ptr(), stream)
     if wait:
         handle.step_streamed(*args)
         return None
