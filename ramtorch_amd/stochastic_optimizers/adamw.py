@@ -377,6 +377,10 @@ class AdamW(Optimizer):
         tensors -- the explicit-noise test mode (every stepped bf16 array needs one).
         ``debug_out``: optional ``{param: (p32, m32, v32)}`` fp32 GPU tensors that
         receive the values before rounding.
+
+        An error raised before the first launch (a sparse or unsupported gradient,
+        tensors on different GPUs, an option combination that is not implemented)
+        leaves every ``state["step"]`` and every tensor as it was.
         """
         loss = None
         if closure is not None:
@@ -388,9 +392,30 @@ class AdamW(Optimizer):
 
         recs = self._records()
         self.finish_early_steps()  # updates started from the backward hook must have landed
-        early = self._stepped_early
         if noise is None and getattr(self, "noise_source", "philox") == "reference":
-            noise = self._reference_noise(grads, early)
+            noise = self._reference_noise(grads, self._stepped_early)
+        # Every step count this call advances is noted, so that they can be put back:
+        # (state, old value) from the Python loop, (states, status bytes) from the C++ gatherer.
+        journal: list = []
+        launched = [False]
+        try:
+            with torch.no_grad():
+                self._step_impl(recs, noise, debug_out, grads, journal, launched)
+        except BaseException:
+            if not launched[0]:
+                for entry in reversed(journal):
+                    if len(entry) == 2:
+                        entry[0]["step"] = entry[1]
+                    else:
+                        states, status, written = entry
+                        for k in np.flatnonzero(status == written):
+                            states[int(k)]["step"] -= 1
+            raise
+        self._stepped_early.clear()
+        return loss
+
+    def _step_impl(self, recs, noise, debug_out, grads, journal, launched) -> None:
+        early = self._stepped_early
         scalars: List[N.RtScalars] = []
         scalar_key: Dict[tuple, int] = {}
         # plain lane: tensors wholly on one GPU, contiguous, nothing special -> columns only
@@ -411,141 +436,154 @@ class AdamW(Optimizer):
             gather = G.module()
         gathered: Dict[int, list] = {}    # dev -> [descriptor buffer, rows used]
 
-        with torch.no_grad():
-            for gi, group in enumerate(self.param_groups):
-                beta1, beta2 = group["betas"]
-                lr, eps, wd, cen = group["lr"], group["eps"], group["weight_decay"], group["centralization"]
-                row = recs[gi]
-                last_step, last_si = None, -1
-                plist = group["params"]
-                work = enumerate(plist)
-                if gather is not None and cen == 0 and row and row[0].plain and isinstance(plist, list):
-                    dev = row[0].dev
-                    slot = gathered.get(dev)
-                    if slot is None:
-                        slot = gathered[dev] = [self._gather_buffer(dev), 0]
-                    buf, used = slot
-                    status = self._gather_status(len(plist))
-                    n_rows, new_steps = gather.gather_group(
-                        plist, self._state_list(gi), dev, buf.ctypes.data + used * buf.itemsize, len(buf) - used,
-                        status.ctypes.data, len(scalars), row[0].tensor_id)
-                    slot[1] = used + n_rows
-                    for st in new_steps:
-                        scalar_key[(gi, st, lr, beta1, beta2, eps, wd, cen)] = len(scalars)
-                        scalars.append(F.make_scalars(lr, (beta1, beta2), eps, wd, st, centralization=cen,
-                                                      inv_loss_scale=inv_loss_scale))
-                    rest = np.flatnonzero(status[:len(plist)] == gather.PYTHON)
-                    work = ((int(k), plist[int(k)]) for k in rest)
-                for k, p in work:
-                    grad = grads.get(p, p.grad) if grads is not None else p.grad
-                    if grad is None:
-                        continue  # adamw.py:114: skipped, and its step count does not advance
-                    if early and id(p) in early:
-                        continue  # already updated by step_param() during this backward
-                    if grad.is_sparse:
-                        raise RuntimeError("AdamW does not support sparse gradients")  # adamw.py:118-119
-                    r = row[k]
+        for gi, group in enumerate(self.param_groups):
+            beta1, beta2 = group["betas"]
+            lr, eps, wd, cen = group["lr"], group["eps"], group["weight_decay"], group["centralization"]
+            row = recs[gi]
+            last_step, last_si = None, -1
+            plist = group["params"]
+            work = enumerate(plist)
+            if gather is not None and cen == 0 and row and row[0].plain and isinstance(plist, list):
+                dev = row[0].dev
+                slot = gathered.get(dev)
+                if slot is None:
+                    slot = gathered[dev] = [self._gather_buffer(dev), 0]
+                buf, used = slot
+                status = self._gather_status(len(plist))
+                status[:len(plist)] = gather.PYTHON  # nothing written yet, should the call itself fail
+                states = self._state_list(gi)
+                journal.append((states, status[:len(plist)], gather.WRITTEN))
+                n_rows, new_steps = gather.gather_group(
+                    plist, states, dev, buf.ctypes.data + used * buf.itemsize, len(buf) - used,
+                    status.ctypes.data, len(scalars), row[0].tensor_id)
+                journal[-1] = (states, status[:len(plist)].copy(), gather.WRITTEN)
+                slot[1] = used + n_rows
+                for st in new_steps:
+                    scalar_key[(gi, st, lr, beta1, beta2, eps, wd, cen)] = len(scalars)
+                    scalars.append(F.make_scalars(lr, (beta1, beta2), eps, wd, st, centralization=cen,
+                                                  inv_loss_scale=inv_loss_scale))
+                rest = np.flatnonzero(status[:len(plist)] == gather.PYTHON)
+                work = ((int(k), plist[int(k)]) for k in rest)
+            for k, p in work:
+                grad = grads.get(p, p.grad) if grads is not None else p.grad
+                if grad is None:
+                    continue  # adamw.py:114: skipped, and its step count does not advance
+                if early and id(p) in early:
+                    continue  # already updated by step_param() during this backward
+                if grad.is_sparse:
+                    raise RuntimeError("AdamW does not support sparse gradients")  # adamw.py:118-119
+                r = row[k]
+                state = r.state
+                if (r.p is not p or state.get("ema") is not r.m or state.get("ema_squared") is not r.v
+                        or p.data_ptr() != r.p_ptr or r.m.data_ptr() != r.m_ptr or r.v.data_ptr() != r.v_ptr):
+                    r = row[k] = self._make_rec(p, r.tensor_id)
                     state = r.state
-                    if (r.p is not p or state.get("ema") is not r.m or state.get("ema_squared") is not r.v
-                            or p.data_ptr() != r.p_ptr or r.m.data_ptr() != r.m_ptr or r.v.data_ptr() != r.v_ptr):
-                        r = row[k] = self._make_rec(p, r.tensor_id)
-                        state = r.state
-                    step = state["step"] + 1  # adamw.py:177
-                    state["step"] = step
-                    if step != last_step:
-                        key = (gi, step, lr, beta1, beta2, eps, wd, cen)
-                        si = scalar_key.get(key)
-                        if si is None:
-                            si = scalar_key[key] = len(scalars)
-                            scalars.append(F.make_scalars(lr, (beta1, beta2), eps, wd, step, centralization=cen,
-                                                          inv_loss_scale=inv_loss_scale))
-                        last_step, last_si = step, si
-                    si = last_si
-                    dev = r.dev
+                step = state["step"] + 1  # adamw.py:177
+                journal.append((state, state["step"]))
+                state["step"] = step
+                if step != last_step:
+                    key = (gi, step, lr, beta1, beta2, eps, wd, cen)
+                    si = scalar_key.get(key)
+                    if si is None:
+                        si = scalar_key[key] = len(scalars)
+                        scalars.append(F.make_scalars(lr, (beta1, beta2), eps, wd, step, centralization=cen,
+                                                      inv_loss_scale=inv_loss_scale))
+                    last_step, last_si = step, si
+                si = last_si
+                dev = r.dev
 
-                    gcode = dt_code.get(grad.dtype)
-                    if (r.plain and cen == 0 and gcode is not None and grad.is_cuda and grad.is_contiguous()
-                            and grad.device.index == dev and grad.numel() == r.numel
-                            and not (extras and ((noise is not None and p in noise)
-                                                 or (debug_out is not None and p in debug_out)))):
-                        lane = plain.get(dev)
-                        if lane is None:
-                            lane = plain[dev] = ([], [], [], [], [], [])
-                        lane[0].append(r); lane[1].append(grad); lane[2].append(grad.data_ptr())
-                        lane[3].append(gcode); lane[4].append(step); lane[5].append(si)
-                        continue
-
-                    # ---- general lane ----
-                    arrays = []
-                    for t in (p.data, r.m, r.v):
-                        if t.is_cuda and t.device.index != dev:
-                            raise RuntimeError("param and optimizer states live on different GPUs")
-                        if not t.is_contiguous():
-                            c = t.contiguous()
-                            writeback.append((t, c))
-                            t = c
-                        arrays.append(t)
-                    g = grad.detach()
-                    if g.is_cuda and g.device.index != dev:
-                        g = g.to(f"cuda:{dev}")
-                    if not g.is_contiguous():
-                        g = g.contiguous()
-                    if g.dtype not in (torch.bfloat16, torch.float32, torch.float16):
-                        g = g.to(torch.float32)  # adamw.py:167 upcasts every gradient to fp32
-                    e = F.Entry(p=arrays[0], g=g, m=arrays[1], v=arrays[2], step=step, scalars_idx=si,
-                                tensor_id=r.tensor_id)
-                    if cen != 0:
-                        if self.max_grad_norm is not None:
-                            raise NotImplementedError("centralization together with max_grad_norm")
-                        if not g.is_cuda:
-                            g = g.to(f"cuda:{dev}", non_blocking=True)
-                            e.g = g
-                        # adamw.py:179-184: mean over every dim but the first (all dims for 0-d / 1-d)
-                        rows = g.shape[0] if g.dim() >= 2 else 1
-                        row_len = g.numel() // rows if rows else 0
-                        if g.numel():
-                            with torch.cuda.device(dev):
-                                e.row_mean = F.row_means(_handle(dev), g, rows, row_len, inv_loss_scale)
-                            e.row_len = row_len
-                    if noise is not None and p in noise:
-                        e.noise = tuple(noise[p])
-                    if debug_out is not None and p in debug_out:
-                        e.dbg = tuple(debug_out[p])
-                    on_gpu = e.p.is_cuda and e.g.is_cuda and e.m.is_cuda and e.v.is_cuda
-                    (resident if on_gpu else streamed).setdefault(dev, []).append(e)
-
-            explicit = noise is not None
-            for dev in sorted(set(plain) | set(resident) | set(streamed) | set(gathered)):
-                h = _handle(dev)
-                with torch.cuda.device(dev):
-                    res, stm = resident.get(dev, []), streamed.get(dev, [])
+                gcode = dt_code.get(grad.dtype)
+                if (r.plain and cen == 0 and gcode is not None and grad.is_cuda and grad.is_contiguous()
+                        and grad.device.index == dev and grad.numel() == r.numel
+                        and not (extras and ((noise is not None and p in noise)
+                                             or (debug_out is not None and p in debug_out)))):
                     lane = plain.get(dev)
-                    descs = self._plain_descs(dev, lane) if lane is not None else None
-                    if dev in gathered and gathered[dev][1]:
-                        d0 = gathered[dev][0][:gathered[dev][1]]
-                        descs = d0 if descs is None else np.concatenate([d0, descs])
-                    if res:
-                        d2 = F.pack_descs(res, streamed=False)
-                        descs = d2 if descs is None else np.concatenate([descs, d2])
-                    clip = skip = None
+                    if lane is None:
+                        lane = plain[dev] = ([], [], [], [], [], [])
+                    lane[0].append(r); lane[1].append(grad); lane[2].append(grad.data_ptr())
+                    lane[3].append(gcode); lane[4].append(step); lane[5].append(si)
+                    continue
+
+                # ---- general lane ----
+                arrays = []
+                for t in (p.data, r.m, r.v):
+                    if t.is_cuda and t.device.index != dev:
+                        raise RuntimeError("param and optimizer states live on different GPUs")
+                    F.dtype_code(t.dtype, "param")  # an unsupported dtype must raise before anything is launched
+                    if not t.is_contiguous():
+                        c = t.contiguous()
+                        writeback.append((t, c))
+                        t = c
+                    arrays.append(t)
+                g = grad.detach()
+                if g.is_cuda and g.device.index != dev:
+                    g = g.to(f"cuda:{dev}")
+                if not g.is_contiguous():
+                    g = g.contiguous()
+                if g.dtype not in (torch.bfloat16, torch.float32, torch.float16):
+                    g = g.to(torch.float32)  # adamw.py:167 upcasts every gradient to fp32
+                if self.max_grad_norm is not None and not g.is_cuda:
+                    # the global norm is taken on the GPU: a host gradient is shipped once, here, and
+                    # the update then reads the device copy
+                    g = g.to(f"cuda:{dev}", non_blocking=True)
+                e = F.Entry(p=arrays[0], g=g, m=arrays[1], v=arrays[2], step=step, scalars_idx=si,
+                            tensor_id=r.tensor_id)
+                if cen != 0:
                     if self.max_grad_norm is not None:
-                        if stm:
-                            raise NotImplementedError("max_grad_norm with host-resident params or states")
-                        gl = (lane[1] if lane is not None else []) + [e.g for e in res]
-                        out = F.grad_norm(h, gl, inv_loss_scale=inv_loss_scale, max_norm=self.max_grad_norm)
-                        self.last_grad_norm = out
-                        clip, skip = out[1:2], out[2:3]
-                    if descs is not None:
-                        F.launch_resident(h, descs, scalars, seed=self.seed, explicit_noise=explicit, clip_coef=clip,
-                                          skip=skip)
-                    if stm:
-                        chunk_elems = max(8, (self.stream_chunk_bytes // 2) // 8 * 8)
-                        F.step_streamed(h, stm, scalars, seed=self.seed, explicit_noise=explicit,
-                                        chunk_elems=chunk_elems)
-            for dst, tmp in writeback:
-                dst.copy_(tmp)
-        early.clear()
-        return loss
+                        raise NotImplementedError("centralization together with max_grad_norm")
+                    if not g.is_cuda:
+                        g = g.to(f"cuda:{dev}", non_blocking=True)
+                        e.g = g
+                    # adamw.py:179-184: mean over every dim but the first (all dims for 0-d / 1-d)
+                    rows = g.shape[0] if g.dim() >= 2 else 1
+                    row_len = g.numel() // rows if rows else 0
+                    if g.numel():
+                        with torch.cuda.device(dev):
+                            e.row_mean = F.row_means(_handle(dev), g, rows, row_len, inv_loss_scale)
+                        e.row_len = row_len
+                if noise is not None and p in noise:
+                    e.noise = tuple(noise[p])
+                if debug_out is not None and p in debug_out:
+                    e.dbg = tuple(debug_out[p])
+                on_gpu = e.p.is_cuda and e.g.is_cuda and e.m.is_cuda and e.v.is_cuda
+                (resident if on_gpu else streamed).setdefault(dev, []).append(e)
+
+        # ---- everything that can still raise for a bad argument happens before the first launch
+        explicit = noise is not None
+        work_by_dev = []
+        for dev in sorted(set(plain) | set(resident) | set(streamed) | set(gathered)):
+            res, stm = resident.get(dev, []), streamed.get(dev, [])
+            lane = plain.get(dev)
+            descs = self._plain_descs(dev, lane) if lane is not None else None
+            if dev in gathered and gathered[dev][1]:
+                d0 = gathered[dev][0][:gathered[dev][1]]
+                descs = d0 if descs is None else np.concatenate([d0, descs])
+            if res:
+                d2 = F.pack_descs(res, streamed=False)
+                descs = d2 if descs is None else np.concatenate([descs, d2])
+            stm_descs = F.pack_descs(stm, streamed=True) if stm else None
+            work_by_dev.append((dev, lane, res, stm, descs, stm_descs))
+
+        for dev, lane, res, stm, descs, stm_descs in work_by_dev:
+            h = _handle(dev)
+            with torch.cuda.device(dev):
+                clip = skip = None
+                if self.max_grad_norm is not None:
+                    # one norm over every gradient of the step, wherever its parameter lives
+                    gl = (lane[1] if lane is not None else []) + [e.g for e in res] + [e.g for e in stm]
+                    out = F.grad_norm(h, gl, inv_loss_scale=inv_loss_scale, max_norm=self.max_grad_norm)
+                    self.last_grad_norm = out
+                    clip, skip = out[1:2], out[2:3]
+                launched[0] = True
+                if descs is not None:
+                    F.launch_resident(h, descs, scalars, seed=self.seed, explicit_noise=explicit, clip_coef=clip,
+                                      skip=skip)
+                if stm:
+                    chunk_elems = max(8, (self.stream_chunk_bytes // 2) // 8 * 8)
+                    F.step_streamed(h, stm, scalars, seed=self.seed, explicit_noise=explicit,
+                                    chunk_elems=chunk_elems, clip_coef=clip, skip=skip, descs=stm_descs)
+        for dst, tmp in writeback:
+            dst.copy_(tmp)
 
     def _reference_noise(self, grads, early) -> dict:
         """The reference's own rounding noise for every parameter about to step: a fresh

@@ -573,3 +573,87 @@ def test_deepcopied_optimizer_steps_like_the_original():
         assert nmis(p.detach(), q.detach()) == 0
         assert nmis(opt.state[p]["ema"], twin.state[q]["ema"]) == 0
         assert opt.state[p]["step"] == twin.state[q]["step"] == 2
+
+
+@pytest.mark.parametrize("n_params", [4, 300])  # 300: the C++ gatherer has advanced step counts before the error
+@pytest.mark.parametrize("kind", ["sparse", "centralization+clip", "bad dtype"])
+def test_a_step_that_raises_leaves_step_counts_and_tensors_untouched(n_params, kind):
+    """The reference raises before it touches the offending tensor (adamw.py:118-119); here whatever
+    the step had already counted for the tensors before it is put back."""
+    shapes = [(16, 8)] * (n_params - 1) + [(10, 4)]
+    ps, grads = _make_params(shapes, 5000)
+    kw = {}
+    if kind == "bad dtype":
+        ps[-1] = torch.nn.Parameter(torch.zeros(10, 4, device="cuda", dtype=torch.float8_e4m3fn), requires_grad=False)
+    groups = [{"params": ps[:-1]}, {"params": ps[-1:]}]
+    if kind == "centralization+clip":
+        groups[1]["centralization"] = 0.5
+        kw["max_grad_norm"] = 1.0
+    opt = ramtorch_amd.AdamW(groups, storage_device="cuda", dtype=torch.bfloat16, **kw)
+    for p, g in zip(ps[:-1], grads):
+        p.grad = g
+    opt.step()  # one good step first (the last parameter has no gradient yet), so that the counts are not all zero
+    torch.cuda.synchronize()
+    snap = [(p.detach().clone(), opt.state[p]["ema"].clone(), opt.state[p]["ema_squared"].clone()) for p in ps[:-1]]
+    steps = [opt.state[p]["step"] for p in ps]
+    if kind == "sparse":
+        ps[-1].grad = torch.sparse_coo_tensor(torch.tensor([[1], [2]]), torch.tensor([1.0]), (10, 4)).cuda().bfloat16()
+        err = RuntimeError
+    elif kind == "bad dtype":
+        ps[-1].grad = torch.zeros(10, 4, device="cuda", dtype=torch.float8_e4m3fn)
+        err = NotImplementedError
+    else:
+        ps[-1].grad = grads[-1]
+        err = NotImplementedError
+    with pytest.raises(err):
+        opt.step()
+    torch.cuda.synchronize()
+    assert [opt.state[p]["step"] for p in ps] == steps
+    for p, (p0, m0, v0) in zip(ps[:-1], snap):
+        assert nmis(p.detach(), p0) == 0 and nmis(opt.state[p]["ema"], m0) == 0
+        assert nmis(opt.state[p]["ema_squared"], v0) == 0
+    # and the optimizer still steps once the offending gradient is gone
+    ps[-1].grad = None
+    opt.step()
+    assert [opt.state[p]["step"] for p in ps[:-1]] == [s + 1 for s in steps[:-1]]
+
+
+def test_short_sqrt_sequence_equals_sqrtf_on_its_whole_domain():
+    """The update kernels' sqrt for wavefronts whose second moments all lie in [2^-96, inf) against the
+    compiler's correctly rounded sqrtf, on every one of the 1 879 048 192 floats of that range."""
+    h = N.Handle(0)
+    try:
+        assert h.selftest_sqrt() == 0
+    finally:
+        h.close()
+
+
+def test_zeros_denormals_and_tiny_second_moments_take_the_full_sqrt():
+    """Wavefronts with a zero, a denormal or a tiny second moment leave the short sqrt path; both paths
+    must give the oracle's bits, also side by side in one launch (fp32 states carry the small values)."""
+    n = 64 * 8 * 6 + 24
+    rng = np.random.default_rng(3)
+    p = rng.normal(0, 0.02, n).astype(np.float32)
+    g = np.zeros(n, np.float32)
+    m = rng.normal(0, 1e-4, n).astype(np.float32)
+    v = (rng.normal(0, 1e-3, n).astype(np.float32)) ** 2
+    v[512:1024] = 0.0                                   # a whole wavefront of zeros
+    v[1024 + 7] = np.float32(1e-40)                     # one denormal in an otherwise ordinary wavefront
+    v[1536:2048] = np.float32(2.0 ** -100)              # tiny but normal
+    v[2048 + 5] = np.float32(np.inf)
+    g[2560:] = rng.normal(0, 1e-3, n - 2560).astype(np.float32)
+    P, G, M, V = (torch.from_numpy(a.copy()).cuda() for a in (p, g, m, v))
+    h = N.Handle(0)
+    try:
+        e = F.Entry(p=P, g=G, m=M, v=V, step=7, scalars_idx=0, tensor_id=0)
+        F.step_resident(h, [e], [F.make_scalars(step=7, **HP0)], seed=5, explicit_noise=False)
+        torch.cuda.synchronize()
+    finally:
+        h.close()
+    po, mo, vo = p.copy(), m.copy(), v.copy()
+    oracle.step_tensor(po, g, mo, vo, oracle.scalars_from_hparams(step=7, **HP0), p_dtype=oracle.DT_F32,
+                       g_dtype=oracle.DT_F32, m_dtype=oracle.DT_F32, v_dtype=oracle.DT_F32, seed=5, step=7, tensor_id=0)
+    for name, t, a in (("p", P, po), ("m", M, mo), ("v", V, vo)):
+        got, want = t.cpu().numpy().view(np.uint32), a.view(np.uint32)
+        both_nan = np.isnan(t.cpu().numpy()) & np.isnan(a)
+        assert ((got == want) | both_nan).all(), name

@@ -294,3 +294,50 @@ def test_load_state_dict_restores_pinned_host_states():
         opt.step()
     assert nmis(ps[0].detach(), ps2[0].detach()) == 0
     assert nmis(a.state[ps[0]]["ema_squared"], st["ema_squared"]) == 0
+
+
+@pytest.mark.parametrize("grads_on", ["cuda", "cpu"])
+def test_max_grad_norm_with_host_resident_params_and_states(grads_on):
+    """Global-norm clip for the offload layout (pinned CPU params and states; gradients on the GPU as
+    config 3 has them, or on the CPU as ramtorch.Linear leaves them): the norm is taken on the GPU over
+    every gradient and the streamed update multiplies by the coefficient.  The norm against a float64
+    sum (1e-6 relative: reduction order), the update bit-exact given the coefficient the kernel used."""
+    shapes = [(300, 70), (4096,), (17,)]
+    ps, gs, refs = [], [], []
+    for i, shp in enumerate(shapes):
+        n = int(np.prod(shp))
+        p, g, _, _ = oracle.synth_inputs(n, 1300 + i)
+        ps.append(torch.nn.Parameter(host16(p).view(shp)))
+        gs.append(g)
+        refs.append([p.copy(), np.zeros(n, np.uint16), np.zeros(n, np.uint16)])
+    opt = ramtorch_amd.AdamW(ps, seed=4, stream_chunk_bytes=8192, max_grad_norm=1e-3, **HP0)
+    for step in (1, 2):
+        gmap = {}
+        for p, g in zip(ps, gs):
+            t = host16(g, pin=False).view(p.shape)
+            gmap[p] = t.cuda() if grads_on == "cuda" else t
+        opt.step(grads=gmap)
+        total = float(opt.last_grad_norm[0])
+        coef = np.float32(opt.last_grad_norm[1].item())
+        want = sum(oracle.grad_sumsq(g, oracle.DT_BF16, 1.0) for g in gs) ** 0.5
+        assert total == pytest.approx(want, rel=1e-6)
+        assert coef < 1.0 and coef == oracle.clip_coef(np.float32(total), 1e-3)
+        sco = oracle.scalars_from_hparams(step=step, apply_clip=True, **HP0)
+        for i, (p, g) in enumerate(zip(ps, gs)):
+            oracle.step_tensor(refs[i][0], g, refs[i][1], refs[i][2], sco, clip_coef=coef, seed=4, step=step,
+                               tensor_id=i)
+            np.testing.assert_array_equal(bits16(p), refs[i][0], err_msg=f"step {step} param {i}")
+            np.testing.assert_array_equal(bits16(opt.state[p]["ema"]), refs[i][1])
+            np.testing.assert_array_equal(bits16(opt.state[p]["ema_squared"]), refs[i][2])
+    # a non-finite gradient: nothing moves
+    snap = [bits16(p).copy() for p in ps]
+    bad = {p: host16(g, pin=False).view(p.shape).cuda() for p, g in zip(ps, gs)}
+    bad[ps[1]][3] = float("inf")
+    opt.step(grads=bad)
+    assert all((bits16(p) == s).all() for p, s in zip(ps, snap))
+    assert opt.last_grad_norm.view(torch.int32)[2].item() == 1
+
+
+def test_host_link_probe_reports_plausible_rates(handle):
+    r = handle.host_link_probe(64 << 20, reps=4)
+    assert all(5.0 < r[k] < 200.0 for k in ("h2d_GBps", "d2h_GBps", "duplex_GBps_each_way")), r
