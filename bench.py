@@ -1,17 +1,20 @@
 #!/usr/bin/env python3
 """Benchmark of the SR-AdamW step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama8b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama8b] [--secondary all|none|a,b,...]
 
 A "step" is one ``AdamW.step()`` over the whole synthetic parameter set, with
-params, grads and both states already resident in HBM (or, for the streamed
-workload, params/states in pinned host memory).  Prints ONE JSON line:
+params, grads and both states already resident in HBM (or, for the host-resident
+workloads, params/states in pinned host memory).  Prints ONE JSON line:
 
-  value      elements updated per second over the K timed steps (wall clock
-             around the steps, device synchronised on both sides)
+  value      elements updated per second over the K timed steps of the main workload
+             (wall clock around the steps, device synchronised on both sides)
   roofline   algorithmic HBM bytes per launch / mean kernel time of the update
              kernel, the kernel time taken with HIP events on the launch stream
              inside the library; peak = 8 TB/s
+  secondary  the other configurations, each measured the same way in the same
+             process with fewer steps (only when the main workload is the
+             default one; ``--secondary none`` leaves them out)
   cpu_baseline  the same ATen op sequence the reference issues
              (ramtorch/stochastic_optimizers/adamw.py:160-222), on CPU tensors
              with all host threads, on a bounded sample; plus the scalar C
@@ -31,10 +34,16 @@ ema~N(0,1e-4), ema_squared=N(0,1e-3)^2, stored bf16):
             backward pass would hand its gradient over (last tensor first), and
             step() only waits: the grad hand-off from ramtorch.Linear's
             post-accumulate hook
+  offload_ref  the same set as the reference's own offload flow leaves it
+            (linear.py:416-427 -> adamw.py:167): pinned CPU params and states
+            and the gradients on the CPU too (in ordinary, not pinned, memory, as
+            ``.to("cpu", non_blocking=True)`` allocates them); 8 bytes per element
+            go up the host link, 6 come down
 """
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import math
 import os
@@ -45,11 +54,18 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch of the update kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this script (scaled by the counters' readings for kernels of known size in the same runs).
-MEASURED_TRAFFIC_BYTES = {"llama8b": 112_546_390_426}
+# HBM bytes per launch of the dominant update kernel.  NOT measured in this run: rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE figures of earlier runs of this script (each scaled by what the same
+# counter reads for a plain kernel of known size in the same run), kept under profiles/.
+OFFLINE_TRAFFIC = {
+    "llama8b": (112_546_390_426, "profiles/sr_adamw_fast_kernel_llama8b_hbm_traffic.txt"),
+}
 HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
 METRIC = "SR-AdamW step: params/sec + achieved HBM GB/s (% of peak), 8B bf16 set, 1 GPU"
+RESIDENT = ("llama8b", "cfg0", "small", "mixed")
+HOST = ("streamed", "hooked", "offload_ref")
+UPDATE_BYTES = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 20}   # per element, update launch only
+STEP_BYTES = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 24, "streamed": 12, "hooked": 12, "offload_ref": 14}
 
 
 # ---- workload shapes -------------------------------------------------------------------------
@@ -118,7 +134,6 @@ def cpu_baseline():
     draws per tensor that the reference pays for.  Bounded sample of the same workload: the
     nine tensors of one transformer layer of the Llama-3-8B-shaped set (218 112 000 elements),
     best of 2 passes after a warm-up pass."""
-    import numpy as np
     import torch
     import oracle
     from oracle import torch_ops
@@ -156,7 +171,7 @@ def cpu_baseline():
 
 
 # ---- GPU workloads ----------------------------------------------------------------------------
-def build_resident(shapes, *, g_dtype, v_dtype, device, seed=1234):
+def build_resident(shapes, *, g_dtype, device, seed=1234):
     import torch
     # parameters first, gradients afterwards: the order a framework allocates them in (model
     # construction, then the backward pass), so a parameter and its gradient are not neighbours
@@ -173,91 +188,69 @@ def build_resident(shapes, *, g_dtype, v_dtype, device, seed=1234):
     return params, grads
 
 
-def main() -> int:
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="llama8b", choices=["llama8b", "cfg0", "small", "mixed", "streamed", "hooked"])
-    ap.add_argument("--layers", type=int, default=32, help="transformer layers of the Llama-shaped set")
-    ap.add_argument("--stream-gb", type=float, default=48.2, help="upper bound on pinned host bytes (streamed)")
-    ap.add_argument("--stream-chunk-mb", type=int, default=256, help="bytes of bf16 per staged chunk and array (streamed)")
-    ap.add_argument("--state-placement", default="auto", choices=["auto", "plain"],
-                    help="AdamW(state_placement=...): 'auto' puts ema and ema_squared into different HBM regions")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--pmc-calibrate", action="store_true",
-                    help="also launch one plain elementwise kernel that reads 1 GiB and writes 1 GiB, so that "
-                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings can be scaled to bytes")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs on ONE GPU; the step needs no exchange between GPUs and a multi-GPU "
-              "figure is not part of it (it would shard by tensor, as ZeRO-1 does). Use --gpus 1.", file=sys.stderr)
-        return 2
+def set_states(opt, params, first_step, warmup, dev):
+    import torch
+    for i, p in enumerate(params):
+        st = opt.state[p]
+        st["step"] = first_step - 1 - warmup
+        # the states stay the tensors the optimizer allocated (and placed); only their contents are set
+        st["ema"].copy_(fill_tensor(p.shape, "m", 1234 + 4 * i + 2, torch.bfloat16, dev))
+        st["ema_squared"].copy_(fill_tensor(p.shape, "v", 1234 + 4 * i + 3, st["ema_squared"].dtype, dev))
 
+
+def timed_steps(one_step, steps, warmup, handle, resident):
+    import torch
+    for _ in range(warmup):
+        one_step()
+    torch.cuda.synchronize()
+    if resident:
+        # the library records a HIP event pair around the update kernels of every launch, on the
+        # launch stream; nothing is read back before the timed region has ended
+        handle.set_timing(True)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        one_step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ks = handle.kernel_ms_history(min(steps, 256)) if resident else []
+    if resident:
+        handle.set_timing(False)
+    return wall * 1e3 / steps, ks
+
+
+def config_of(wl, shapes, total, first_step, explicit):
+    return {"workload": wl, "tensors": len(shapes), "elements": total, "bytes_per_element": STEP_BYTES[wl],
+            "first_timed_step": first_step, "noise": "explicit int16" if explicit else "philox seed 1234",
+            "hparams": {"lr": HP["lr"], "betas": list(HP["betas"]), "eps": HP["eps"],
+                        "weight_decay": HP["weight_decay"]}}
+
+
+def run_resident(wl, args, steps, warmup, *, full):
+    """One resident workload.  ``full``: also the math-free ceilings and the plain-placement comparison."""
     import torch
     import ramtorch_amd
     from ramtorch_amd.stochastic_optimizers import adamw as adamw_mod
 
-    if not torch.cuda.is_available():
-        print("bench.py needs an MI355X", file=sys.stderr)
-        return 1
     dev = "cuda:0"
-    torch.cuda.set_device(0)
-    wl = args.workload
     first_step = 100
-    noise = None
     opt_kw = dict(storage_device="cuda", seed=1234, state_placement=args.state_placement)
-    bytes_per_elem = 14
-    dtype_label = "f32"  # arithmetic type; storage is bf16 (or fp32 for the mixed layout)
+    g_dtype = torch.bfloat16
     if wl == "llama8b":
         shapes = llama3_8b_shapes(args.layers)
-        params, grads = build_resident(shapes, g_dtype=torch.bfloat16, v_dtype=torch.bfloat16, device=dev)
-        state_dtype = torch.bfloat16
     elif wl == "cfg0":
         shapes = [(4096, 4096)]
-        params, grads = build_resident(shapes, g_dtype=torch.bfloat16, v_dtype=torch.bfloat16, device=dev)
-        state_dtype = torch.bfloat16
         first_step = 10
-        bytes_per_elem = 20
     elif wl == "small":
         shapes = small_tensor_shapes()
-        params, grads = build_resident(shapes, g_dtype=torch.bfloat16, v_dtype=torch.bfloat16, device=dev)
-        state_dtype = torch.bfloat16
-    elif wl == "mixed":
+    else:  # mixed
         shapes = llama3_8b_shapes(args.layers)
-        params, grads = build_resident(shapes, g_dtype=torch.float32, v_dtype=torch.float32, device=dev)
-        state_dtype = torch.bfloat16
+        g_dtype = torch.float32
         opt_kw.update(loss_scale=1024.0, max_grad_norm=1.0, ema_squared_dtype=torch.float32)
-        bytes_per_elem = 24
-    else:  # streamed / hooked
-        shapes = llama3_8b_shapes(args.layers)
-        budget = int(args.stream_gb * 1e9)
-        kept, used = [], 0
-        for shp in shapes:
-            if used + 6 * numel(shp) > budget:
-                break
-            kept.append(shp)
-            used += 6 * numel(shp)
-        shapes = kept
-        params, grads = [], []
-        for i, shp in enumerate(shapes):
-            p = fill_tensor(shp, "p", 1234 + 4 * i, torch.bfloat16, dev).cpu().pin_memory()
-            params.append(torch.nn.Parameter(p, requires_grad=False))
-            grads.append(fill_tensor(shp, "g", 1234 + 4 * i + 1, torch.bfloat16, dev))
-        state_dtype = torch.bfloat16
-        opt_kw = dict(storage_device="cpu", seed=1234, stream_chunk_bytes=args.stream_chunk_mb << 20)
-        bytes_per_elem = 12
-        if wl == "hooked":
-            gmap_needed = False
-
+    params, grads = build_resident(shapes, g_dtype=g_dtype, device=dev)
     total = sum(numel(s) for s in shapes)
-    opt = ramtorch_amd.AdamW(params, dtype=state_dtype, **HP, **opt_kw)
-    for i, p in enumerate(params):
-        st = opt.state[p]
-        st["step"] = first_step - 1 - args.warmup
-        # the states stay the tensors the optimizer allocated (and placed); only their contents are set
-        st["ema"].copy_(fill_tensor(p.shape, "m", 1234 + 4 * i + 2, torch.bfloat16, dev))
-        st["ema_squared"].copy_(fill_tensor(p.shape, "v", 1234 + 4 * i + 3, st["ema_squared"].dtype, dev))
+    opt = ramtorch_amd.AdamW(params, dtype=torch.bfloat16, **HP, **opt_kw)
+    set_states(opt, params, first_step, warmup, dev)
+    noise = None
     if wl == "cfg0":
         noise = {params[0]: tuple(torch.randint(-32768, 32768, (4096, 4096), dtype=torch.int16, device=dev,
                                                 generator=torch.Generator(dev).manual_seed(1234 + k))
@@ -270,61 +263,39 @@ def main() -> int:
             p.grad = g
         gmap = None
     torch.cuda.synchronize()
-
     handle = adamw_mod._handle(0)
-    if "RT_MAX_INFLIGHT_CALLS" in os.environ:  # experiment knob: chunks step_param may queue ahead
-        opt.max_inflight_calls = int(os.environ["RT_MAX_INFLIGHT_CALLS"])
-    if "RT_POLL_SECONDS" in os.environ:
-        opt._poll_seconds = float(os.environ["RT_POLL_SECONDS"])
 
-    def one_step():
-        if wl == "hooked":
-            for p, g in zip(reversed(params), reversed(grads)):
-                opt.step_param(p, g)
-            opt.step()
-        else:
-            opt.step(noise=noise, grads=gmap)
-
-    for _ in range(args.warmup):
-        one_step()
-    torch.cuda.synchronize()
-    resident = wl not in ("streamed", "hooked")
-    if resident:
-        # the library records a HIP event pair around the update kernels of every launch, on the
-        # launch stream; nothing is read back before the timed region has ended
-        handle.set_timing(True)
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        one_step()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
-    kernel_times = handle.kernel_ms_history(min(args.steps, 256)) if resident else []
-    if resident:
-        handle.set_timing(False)
-
-    # kernel time of the update launch: mean over the launches of the timed region (the most
-    # recent 256 when there were more), from the event pairs recorded above
-    roofline = None
-    stream_info = None
-    if resident:
-        ks = kernel_times
-        k_ms = sum(ks) / len(ks)
-        # the update launch moves 14 (20 with explicit noise; 20 for the mixed layout, whose
-        # norm pass is a separate launch of 4 B/elem) bytes per element
-        upd_bytes = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 20}[wl] * total
-        achieved = upd_bytes / (k_ms * 1e-3) / 1e9
-        roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                    "frac": achieved / HBM_PEAK_GBPS,
-                    "traffic": MEASURED_TRAFFIC_BYTES.get(wl) if args.layers == 32 else None,
-                    "kernel": "sr_adamw_fast_wide_kernel" if wl == "mixed" else "sr_adamw_fast_kernel",
-                    "kernel_ms": k_ms, "kernel_launches_timed": len(ks), "algorithmic_bytes_per_launch": upd_bytes}
+    ms_per_step, ks = timed_steps(lambda: opt.step(noise=noise, grads=gmap), steps, warmup, handle, True)
+    k_ms = sum(ks) / len(ks)
+    upd_bytes = UPDATE_BYTES[wl] * total
+    achieved = upd_bytes / (k_ms * 1e-3) / 1e9
+    traffic = OFFLINE_TRAFFIC.get(wl) if args.layers == 32 else None
+    roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic[0] if traffic else None,
+                "traffic_source": (f"not measured in this run: rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of an earlier "
+                                   f"run, {traffic[1]}") if traffic else None,
+                "kernel": "sr_adamw_fast_wide_kernel" if wl == "mixed" else "sr_adamw_fast_kernel",
+                "kernel_ms": k_ms, "kernel_launches_timed": len(ks), "algorithmic_bytes_per_launch": upd_bytes}
+    out = {"ms_per_step": ms_per_step, "elements_per_s": total / (ms_per_step * 1e-3),
+           "achieved_GBps_wall": STEP_BYTES[wl] * total / (ms_per_step * 1e-3) / 1e9,
+           "config": config_of(wl, shapes, total, first_step, noise is not None), "roofline": roofline}
+    if full:
+        # The same state tensors allocated one by one, as the reference allocates them, instead of
+        # in two pools placed in different HBM regions: what the placement is worth on this box.
+        if args.state_placement == "auto" and opt.state_placement_report is not None:
+            plain = ramtorch_amd.AdamW(params, dtype=torch.bfloat16, **HP, **dict(opt_kw, state_placement="plain"))
+            for p in params:
+                plain.state[p]["step"] = first_step - 1
+            _, ks2 = timed_steps(lambda: plain.step(noise=noise, grads=gmap), max(3, steps // 4), 2, handle, True)
+            k2 = sum(ks2) / len(ks2)
+            roofline["plain_placement"] = {"kernel_ms": k2, "achieved": upd_bytes / (k2 * 1e-3) / 1e9,
+                                           "frac": upd_bytes / (k2 * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+            del plain
         # What the same traffic pattern reaches with the arithmetic removed (the all-bf16 pattern:
-        # 8 B read + 6 B written per element).  Where the arrays lie in HBM matters (see
-        # ramtorch_amd/placement.py), so it is measured twice: on four fresh buffers allocated
-        # side by side, and on the workload's own largest tensor (p, its gradient and its two
-        # states, where the optimizer placed them).  The probe overwrites what it runs on, which
-        # is why it comes last.
+        # 8 B read + 6 B written per element).  Where the arrays lie in HBM matters, so it is measured
+        # twice: on four fresh buffers allocated side by side, and on the workload's own largest
+        # tensor (p, its gradient and its two states, where the optimizer placed them).  The probe
+        # overwrites what it runs on, which is why it comes last.
         n_probe = 1 << 30
         bufs = [torch.zeros(n_probe, dtype=torch.bfloat16, device=dev) for _ in range(4)]
         torch.cuda.synchronize()
@@ -338,43 +309,87 @@ def main() -> int:
         if n_own >= (1 << 24) and all(a.data_ptr() % 16 == 0 for a in arrs):
             probe_ms = handle.stream_probe(*[a.data_ptr() for a in arrs], n_own, reps=5)
             roofline["pattern_ceiling_GBps"] = 14 * n_own / (probe_ms * 1e-3) / 1e9
-        roofline["frac_of_pattern_ceiling"] = achieved / roofline["pattern_ceiling_GBps"] if wl in ("llama8b", "small") else None
-        roofline["state_placement"] = {"mode": args.state_placement, **(opt.state_placement_report or {})}
-    else:
-        if wl == "streamed":
-            st = handle.streamed_stats()
-        else:  # per-tensor asynchronous calls: the whole step is the unit
-            st = {"bytes_h2d": 6.0 * total, "bytes_d2h": 6.0 * total, "seconds": ms_per_step * 1e-3}
-        stream_info = {"h2d_GBps": st["bytes_h2d"] / st["seconds"] / 1e9, "d2h_GBps": st["bytes_d2h"] / st["seconds"] / 1e9,
-                       "seconds_last_call": st["seconds"], "host_bytes": 6 * total}
-        # same-run pinned-copy peaks with the same chunk size
-        chunk = args.stream_chunk_mb << 20
-        hbuf = torch.empty(chunk, dtype=torch.uint8).pin_memory()
-        dbuf = torch.empty(chunk, dtype=torch.uint8, device=dev)
-        for name, (dst, src) in (("h2d", (dbuf, hbuf)), ("d2h", (hbuf, dbuf))):
-            dst.copy_(src, non_blocking=True)
-            torch.cuda.synchronize()
-            t1 = time.perf_counter()
-            for _ in range(8):
-                dst.copy_(src, non_blocking=True)
-            torch.cuda.synchronize()
-            stream_info[f"pinned_{name}_peak_GBps"] = 8 * chunk / (time.perf_counter() - t1) / 1e9
-        stream_info["h2d_frac_of_peak"] = stream_info["h2d_GBps"] / stream_info["pinned_h2d_peak_GBps"]
-        # both directions at once (what the pipeline does in steady state): two streams, one chunk each way
-        hbuf2 = torch.empty(chunk, dtype=torch.uint8).pin_memory()
-        dbuf2 = torch.empty(chunk, dtype=torch.uint8, device=dev)
-        s_up, s_down = torch.cuda.Stream(), torch.cuda.Stream()
+        roofline["frac_of_pattern_ceiling"] = (achieved / roofline["pattern_ceiling_GBps"]
+                                               if wl in ("llama8b", "small") else None)
+    roofline["state_placement"] = {"mode": args.state_placement, **(opt.state_placement_report or {})}
+    if wl == "mixed":
+        # the norm pass is a launch of its own (4 B per element read); time it apart
+        from ramtorch_amd import functional as F
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        F.grad_norm(handle, grads, inv_loss_scale=1 / 1024, max_norm=1.0)
+        ev[0].record()
+        for _ in range(3):
+            F.grad_norm(handle, grads, inv_loss_scale=1 / 1024, max_norm=1.0)
+        ev[1].record()
         torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        for _ in range(8):
-            with torch.cuda.stream(s_up):
-                dbuf.copy_(hbuf, non_blocking=True)
-            with torch.cuda.stream(s_down):
-                hbuf2.copy_(dbuf2, non_blocking=True)
-        torch.cuda.synchronize()
-        stream_info["pinned_duplex_peak_GBps_each_way"] = 8 * chunk / (time.perf_counter() - t1) / 1e9
-        stream_info["frac_of_duplex_peak"] = stream_info["d2h_GBps"] / stream_info["pinned_duplex_peak_GBps_each_way"]
-        del hbuf2, dbuf2
+        n_ms = ev[0].elapsed_time(ev[1]) / 3
+        roofline["norm_pass"] = {"kernel": "grad_sumsq_kernel", "ms": n_ms, "achieved": 4 * total / (n_ms * 1e-3) / 1e9,
+                                 "frac": 4 * total / (n_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+    del opt, params, grads, gmap, noise
+    gc.collect()
+    torch.cuda.empty_cache()
+    return out
+
+
+def run_host(workloads, args, steps, warmup):
+    """The host-resident workloads, on one set of pinned host arrays (pinning 48 GB takes a while)."""
+    import torch
+    import ramtorch_amd
+    from ramtorch_amd.stochastic_optimizers import adamw as adamw_mod
+
+    dev = "cuda:0"
+    shapes = llama3_8b_shapes(args.layers)
+    budget = int(args.stream_gb * 1e9)
+    kept, used = [], 0
+    for shp in shapes:
+        if used + 6 * numel(shp) > budget:
+            break
+        kept.append(shp)
+        used += 6 * numel(shp)
+    shapes = kept
+    total = sum(numel(s) for s in shapes)
+    t_pin = time.perf_counter()
+    params, grads = [], []
+    for i, shp in enumerate(shapes):
+        p = fill_tensor(shp, "p", 1234 + 4 * i, torch.bfloat16, dev).cpu().pin_memory()
+        params.append(torch.nn.Parameter(p, requires_grad=False))
+        grads.append(fill_tensor(shp, "g", 1234 + 4 * i + 1, torch.bfloat16, dev))
+    opt = ramtorch_amd.AdamW(params, dtype=torch.bfloat16, **HP, storage_device="cpu", seed=1234,
+                             stream_chunk_bytes=args.stream_chunk_mb << 20)
+    set_states(opt, params, 100, warmup * len(workloads), dev)
+    torch.cuda.synchronize()
+    setup_s = time.perf_counter() - t_pin
+    handle = adamw_mod._handle(0)
+    gmap = dict(zip(params, grads))
+    results = {}
+    link = None
+    for wl in workloads:
+        cpu_grads = None
+        if wl == "hooked":
+            def one_step():
+                for p, g in zip(reversed(params), reversed(grads)):
+                    opt.step_param(p, g)
+                opt.step()
+        elif wl == "offload_ref":
+            # gradients where Linear.backward leaves them: ordinary CPU memory
+            cpu_grads = {p: g.to("cpu") for p, g in gmap.items()}
+            one_step = lambda: opt.step(grads=cpu_grads)
+        else:
+            one_step = lambda: opt.step(grads=gmap)
+        ms_per_step, _ = timed_steps(one_step, steps, warmup, handle, False)
+        up = {"streamed": 6.0, "hooked": 6.0, "offload_ref": 8.0}[wl] * total
+        down = 6.0 * total
+        secs = ms_per_step * 1e-3
+        info = {"h2d_GBps": up / secs / 1e9, "d2h_GBps": down / secs / 1e9, "host_bytes_up": up, "host_bytes_down": down}
+        if link is None:
+            # same-run pinned-copy peaks with the same chunk size, each direction alone and both at
+            # once (what the pipeline does in steady state), on the library's own copy streams
+            link = handle.host_link_probe(args.stream_chunk_mb << 20, reps=8)
+        info["pinned_h2d_peak_GBps"] = link["h2d_GBps"]
+        info["pinned_d2h_peak_GBps"] = link["d2h_GBps"]
+        info["pinned_duplex_peak_GBps_each_way"] = link["duplex_GBps_each_way"]
+        info["h2d_frac_of_peak"] = info["h2d_GBps"] / link["h2d_GBps"]
+        info["frac_of_duplex_peak"] = info["d2h_GBps"] / link["duplex_GBps_each_way"]
         if wl == "streamed":
             # per-chunk copy durations of one more step, from events the library records on its copy streams
             handle.set_timing(True)
@@ -384,37 +399,111 @@ def main() -> int:
             if tl:
                 h2d = [r[1] - r[0] for r in tl]
                 d2h = [r[3] - r[2] for r in tl]
-                stream_info["chunks"] = len(tl)
-                stream_info["h2d_chunk_ms"] = {"first": h2d[0], "median": sorted(h2d)[len(h2d) // 2], "max": max(h2d)}
-                stream_info["d2h_chunk_ms"] = {"median": sorted(d2h)[len(d2h) // 2], "max": max(d2h), "last": d2h[-1]}
-                stream_info["pipeline_ms"] = tl[-1][3] - tl[0][0]
-        roofline = {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": None,
-                    "traffic": None, "note": "host-link bound; see host_link"}
+                info["chunks"] = len(tl)
+                info["h2d_chunk_ms"] = {"first": h2d[0], "median": sorted(h2d)[len(h2d) // 2], "max": max(h2d)}
+                info["d2h_chunk_ms"] = {"median": sorted(d2h)[len(d2h) // 2], "max": max(d2h), "last": d2h[-1]}
+                info["pipeline_ms"] = tl[-1][3] - tl[0][0]
+        del cpu_grads
+        results[wl] = {"ms_per_step": ms_per_step, "elements_per_s": total / secs,
+                       "config": config_of(wl, shapes, total, 100, False), "host_link": info,
+                       "roofline": {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                                    "frac": None, "traffic": None, "note": "host-link bound; see host_link"}}
+    for r in results.values():
+        r["setup_seconds"] = setup_s
+    del opt, params, grads, gmap
+    gc.collect()
+    torch.cuda.empty_cache()
+    return results
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="llama8b", choices=list(RESIDENT + HOST))
+    ap.add_argument("--secondary", default=None,
+                    help="'all', 'none' or a comma-separated list of workloads measured after the main one "
+                         "(default: all when the main workload is llama8b, none otherwise)")
+    ap.add_argument("--layers", type=int, default=32, help="transformer layers of the Llama-shaped set")
+    ap.add_argument("--stream-gb", type=float, default=48.2, help="upper bound on pinned host bytes (host-resident workloads)")
+    ap.add_argument("--stream-chunk-mb", type=int, default=256, help="bytes of bf16 per staged chunk and array")
+    ap.add_argument("--state-placement", default="auto", choices=["auto", "plain"],
+                    help="AdamW(state_placement=...): 'auto' puts ema and ema_squared into different HBM regions")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-calibrate", action="store_true",
+                    help="also launch one plain elementwise kernel that reads 1 GiB and writes 1 GiB, so that "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings can be scaled to bytes")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; the step needs no exchange between GPUs and a multi-GPU "
+              "figure is not part of it (it would shard by tensor, as ZeRO-1 does). Use --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X", file=sys.stderr)
+        return 1
+    torch.cuda.set_device(0)
+    wl = args.workload
+    everything = [w for w in RESIDENT + HOST if w != wl]
+    if args.secondary is None:
+        secondary = everything if wl == "llama8b" else []
+    elif args.secondary == "all":
+        secondary = everything
+    elif args.secondary == "none":
+        secondary = []
+    else:
+        secondary = [w for w in args.secondary.split(",") if w]
+        bad = [w for w in secondary if w not in RESIDENT + HOST]
+        if bad:
+            print(f"bench.py: unknown workload(s) {bad}", file=sys.stderr)
+            return 2
+
+    t_begin = time.perf_counter()
+    if wl in RESIDENT:
+        main_res = run_resident(wl, args, args.steps, args.warmup, full=True)
+    else:
+        main_res = run_host([wl], args, args.steps, args.warmup)[wl]
 
     if args.pmc_calibrate:
-        x = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        x = torch.ones(1 << 28, dtype=torch.float32, device="cuda:0")
         y = torch.empty_like(x)
         torch.cuda.synchronize()
         torch.add(x, 1.0, out=y)  # vectorized_elementwise_kernel: 2^30 bytes in, 2^30 bytes out
         torch.cuda.synchronize()
         del x, y
 
+    sec = {}
+    # fewer steps for the secondary configurations: the whole default run has to fit a few minutes
+    for w in [w for w in secondary if w in RESIDENT]:
+        k = {"cfg0": max(args.steps, 20), "small": max(args.steps, 20)}.get(w, max(3, min(args.steps, 10)))
+        r = run_resident(w, args, k, min(args.warmup, 3), full=False)
+        r["steps"] = k
+        sec[w] = r
+    host = [w for w in secondary if w in HOST]
+    if host:
+        k = max(2, min(args.steps, 3))
+        for w, r in run_host(host, args, k, 1).items():
+            r["steps"] = k
+            sec[w] = r
+
     out = {
-        "metric": METRIC, "value": total / (ms_per_step * 1e-3), "unit": "elements/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": dtype_label, "data": "synthetic",
-        "config": {"workload": wl, "tensors": len(shapes), "elements": total, "bytes_per_element": bytes_per_elem,
-                   "first_timed_step": first_step, "noise": "explicit int16" if noise else "philox seed 1234",
-                   "hparams": {"lr": HP["lr"], "betas": list(HP["betas"]), "eps": HP["eps"],
-                               "weight_decay": HP["weight_decay"]}},
-        "achieved_GBps_wall": bytes_per_elem * total / (ms_per_step * 1e-3) / 1e9,
-        "roofline": roofline,
+        "metric": METRIC, "value": main_res["elements_per_s"], "unit": "elements/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32",  # arithmetic type; storage is bf16 (or fp32 for the mixed layout)
+        "data": "synthetic", "config": main_res["config"],
+        "achieved_GBps_wall": main_res.get("achieved_GBps_wall"),
+        "roofline": main_res["roofline"],
     }
-    if stream_info:
-        out["host_link"] = stream_info
+    if "host_link" in main_res:
+        out["host_link"] = main_res["host_link"]
+    if sec:
+        out["secondary"] = sec
+    out["gpu_seconds_total"] = time.perf_counter() - t_begin
     if not args.no_cpu_baseline:
-        del params, grads, opt, gmap
-        torch.cuda.empty_cache()
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out), flush=True)
     return 0
