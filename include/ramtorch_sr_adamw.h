@@ -189,6 +189,22 @@ int rt_grad_norm(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, float in
                  float max_norm, void* d_out, void* stream);
 
 /*
+ * rt_grad_norm for callers that cannot allocate device memory: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has
+ * no counterpart in the reference.  Same arguments, same result bit for bit,
+ * but the per-workgroup partial sums and the gradient table live in a fixed
+ * 144 KiB device array that is part of the library's code object (one copy per
+ * GPU, held until the process ends), the table travels there as kernel
+ * arguments, and the call performs no hipMalloc / hipFree / hipHostMalloc.
+ * Limit: at most 4096 gradients with numel != 0 per call; more returns
+ * RT_EUNSUPPORTED.  Every call on one GPU uses that GPU's one array: calls
+ * that overlap on a GPU (different streams or handles) race; calls queued on
+ * one stream are safe.
+ */
+int rt_grad_norm_static(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, float inv_loss_scale,
+                        float max_norm, void* d_out, void* stream);
+
+/*
  * Row means of g over all dims but the first, for gradient centralization
  * (adamw.py:179-184): d_row_mean[r] = mean(g[r, ...]) in fp32.
  */

@@ -29,7 +29,7 @@ EXPORTS = (
     "rt_grad_norm", "rt_row_means", "rt_sr_copy", "rt_set_timing", "rt_last_kernel_ms", "rt_kernel_ms_history", "rt_streamed_stats",
     "rt_stream_probe", "rt_streamed_timeline", "rt_streamed_plan",
     "rt_step_streamed_async", "rt_streamed_wait", "rt_streamed_completed",
-    "rt_host_link_probe", "rt_selftest_sqrt",
+    "rt_grad_norm_static", "rt_host_link_probe", "rt_selftest_sqrt",
 )
 
 
@@ -119,6 +119,8 @@ def lib() -> ctypes.CDLL:
     L.rt_step_streamed.argtypes = [vp, descs, u32, scal, u32, u64, i32, u64, vp, vp, vp]
     L.rt_grad_norm.restype = i32
     L.rt_grad_norm.argtypes = [vp, descs, u32, ctypes.c_float, ctypes.c_float, vp, vp]
+    L.rt_grad_norm_static.restype = i32
+    L.rt_grad_norm_static.argtypes = [vp, descs, u32, ctypes.c_float, ctypes.c_float, vp, vp]
     L.rt_host_link_probe.restype = i32
     L.rt_host_link_probe.argtypes = [vp, u64, i32, ctypes.POINTER(ctypes.c_double)]
     L.rt_selftest_sqrt.restype = i32
@@ -226,6 +228,11 @@ class Handle:
     def grad_norm(self, descs, n, inv_loss_scale, max_norm, d_out, stream=0):
         with self._lock:
             check(lib().rt_grad_norm(self.ptr, descs, n, inv_loss_scale, max_norm, d_out, stream))
+
+    def grad_norm_static(self, descs, n, inv_loss_scale, max_norm, d_out, stream=0):
+        """rt_grad_norm without any device allocation (at most 4096 non-empty gradients)."""
+        with self._lock:
+            check(lib().rt_grad_norm_static(self.ptr, descs, n, inv_loss_scale, max_norm, d_out, stream))
 
     def host_link_probe(self, nbytes: int, reps: int = 8):
         """Pinned-copy rates of the host link in GB/s: host to device, device to host, each way with both at once."""

@@ -12,6 +12,7 @@
 #include <cstdint>
 #include <cstring>
 #include <map>
+#include <mutex>
 #include <new>
 #include <thread>
 #include <vector>
@@ -109,11 +110,30 @@ struct Streamed {
 
 }  // namespace
 
+// ---------------------------------------------------------------------------
+// Device memory of the entry point that allocates nothing (rt_grad_norm_static): the per-workgroup
+// partial sums and the gradient table, in one array that is part of the loaded code object -- every
+// GPU the library runs on holds its own copy at its own address until the process ends.  Host code
+// never uses the array's name as an address: rt_create asks for the address once per device
+// (hipGetSymbolAddress) and everything below works with that pointer.
+// ---------------------------------------------------------------------------
+namespace {
+constexpr uint32_t kStaticMaxTensors = 4096;  // non-empty gradients per rt_grad_norm_static call
+constexpr size_t kStaticPartialsBytes = kNormPartials * sizeof(double);
+constexpr size_t kStaticScratchBytes = kStaticPartialsBytes + kStaticMaxTensors * sizeof(NormEntry);  // 144 KiB
+constexpr int kMaxDevices = 64;
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static void* g_scratch_ptr[kMaxDevices];  // device -> address of that device's copy of `scratch`
+static std::mutex g_scratch_mutex;
+
 struct rt_handle {
     int device = 0;
     TableSlot slots[kSlots];
     uint64_t slot_counter = 0;
     DevBuf norm_partials;
+    void* static_scratch = nullptr;       // this device's copy of `scratch`
+    std::vector<NormEntry> norm_entries;  // host image of the table of rt_grad_norm_static
     std::vector<uint8_t> image;  // scratch for building a table image
     std::vector<DevTensor> tens;
     std::vector<uint32_t> ranges;       // first unit of each tensor of the fast kernel
@@ -596,9 +616,22 @@ int rt_create(int device, rt_handle** out) {
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(RT_EUNSUPPORTED, "device %d is %s; this library is built for gfx950 only", device,
                     prop.gcnArchName);
+    if (device >= kMaxDevices) return fail(RT_EUNSUPPORTED, "device %d: at most %d devices", device, kMaxDevices);
+    void* scratch_ptr = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (!g_scratch_ptr[device]) {
+            void* ptr = nullptr;
+            HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));  // with `device` current: its own copy
+            g_scratch_ptr[device] = ptr;
+        }
+        scratch_ptr = g_scratch_ptr[device];
+    }
     rt_handle* h = new (std::nothrow) rt_handle();
     if (!h) return fail(RT_ENOMEM, "out of host memory");
     h->device = device;
+    h->static_scratch = scratch_ptr;
+    h->norm_entries.reserve(kStaticMaxTensors);
     hipError_t e = hipSuccess;
     for (int i = 0; i < kSlots && e == hipSuccess; ++i)
         e = hipEventCreateWithFlags(&h->slots[i].done, hipEventDisableTiming);
@@ -766,6 +799,70 @@ int rt_grad_norm(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, float in
     }
     hipLaunchKernelGGL(grad_norm_finish_kernel, dim3(1), dim3(kThreads), 0, stream,
                        (const double*)h->norm_partials.ptr, grid, max_norm, (float*)d_out);
+    HIP_TRY(hipGetLastError());
+    return RT_OK;
+}
+
+int rt_grad_norm_static(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, float inv_loss_scale, float max_norm,
+                        void* d_out, void* stream_) {
+    if (!h) return fail(RT_EINVAL, "handle is NULL");
+    if (!d_out || ((uintptr_t)d_out & 15u)) return fail(RT_EINVAL, "d_out must be a 16-byte aligned device pointer");
+    if (n > 0 && !descs) return fail(RT_EINVAL, "descs is NULL");
+    if (!h->static_scratch) return fail(RT_EHIP, "the static scratch array has no address on device %d", h->device);
+    hipStream_t stream = (hipStream_t)stream_;
+    HIP_TRY(hipSetDevice(h->device));
+    // Chunks are numbered as the chunk list of rt_grad_norm orders them: every whole chunk of the
+    // 16-byte aligned gradients first, then all other chunks, each in tensor order.
+    std::vector<NormEntry>& tab = h->norm_entries;  // capacity reserved by rt_create
+    tab.clear();
+    uint64_t n_whole = 0, n_rest = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        const rt_tensor_desc& d = descs[i];
+        if (d.g_dtype > RT_DT_F16) return fail(RT_EINVAL, "tensor %u: g_dtype %d unknown", i, d.g_dtype);
+        if (d.host_mask) return fail(RT_EINVAL, "tensor %u: host_mask set (grads must be device resident)", i);
+        if (d.numel == 0) continue;
+        if (!d.g) return fail(RT_EINVAL, "tensor %u: g is NULL", i);
+        if ((uintptr_t)d.g % dtype_size(d.g_dtype))
+            return fail(RT_EINVAL, "tensor %u: g not aligned to its element size", i);
+        if (d.numel / kChunkElems >= 0xFFFFFFFFull) return fail(RT_EUNSUPPORTED, "tensor %u: numel too large", i);
+        if (tab.size() >= kStaticMaxTensors)
+            return fail(RT_EUNSUPPORTED,
+                        "rt_grad_norm_static takes at most %u non-empty gradients per call (its table is a fixed "
+                        "device array); use rt_grad_norm", kStaticMaxTensors);
+        const uint64_t chunks = (d.numel + kChunkElems - 1) / kChunkElems;
+        const uint64_t whole = ((uintptr_t)d.g & 15u) == 0 ? d.numel / kChunkElems : 0;
+        NormEntry e;
+        e.g = (uint64_t)d.g;
+        e.numel = d.numel;
+        e.first_whole = (uint32_t)n_whole;
+        e.first_rest = (uint32_t)n_rest;
+        e.n_whole = (uint32_t)whole;
+        e.dtype = d.g_dtype;
+        tab.push_back(e);
+        n_whole += whole;
+        n_rest += chunks - whole;
+        if (n_whole + n_rest > kMaxGrid) return fail(RT_EUNSUPPORTED, "too many elements in one call");
+    }
+    double* partials = (double*)h->static_scratch;
+    NormEntry* table = (NormEntry*)((uint8_t*)h->static_scratch + kStaticPartialsBytes);
+    const uint32_t n_chunks = (uint32_t)(n_whole + n_rest);
+    const uint32_t grid = std::min<uint32_t>(kNormPartials, n_chunks);
+    // the table reaches the device array as kernel arguments, a slice per launch
+    for (uint32_t first = 0; first < tab.size(); first += kNormEntriesPerWrite) {
+        NormEntrySlice slice;
+        const uint32_t count = std::min<uint32_t>(kNormEntriesPerWrite, (uint32_t)tab.size() - first);
+        memcpy(slice.e, tab.data() + first, count * sizeof(NormEntry));
+        hipLaunchKernelGGL(norm_table_write_kernel, dim3(1), dim3(kNormEntriesPerWrite), 0, stream, table, first,
+                           count, slice);
+        HIP_TRY(hipGetLastError());
+    }
+    if (n_chunks != 0) {
+        hipLaunchKernelGGL(grad_sumsq_table_kernel, dim3(grid), dim3(kThreads), 0, stream, (const NormEntry*)table,
+                           (uint32_t)tab.size(), (uint32_t)n_whole, n_chunks, inv_loss_scale, partials);
+        HIP_TRY(hipGetLastError());
+    }
+    hipLaunchKernelGGL(grad_norm_finish_kernel, dim3(1), dim3(kThreads), 0, stream, (const double*)partials, grid,
+                       max_norm, (float*)d_out);
     HIP_TRY(hipGetLastError());
     return RT_OK;
 }

@@ -1085,6 +1085,61 @@ __global__ __launch_bounds__(kThreads) void grad_sumsq_kernel(const DevTensor* _
     if (threadIdx.x == 0) partials[blockIdx.x] = total;
 }
 
+// ---------------------------------------------------------------------------
+// The same pass without a chunk list, for the entry point that allocates
+// nothing: the only table is one NormEntry per gradient, small enough to live
+// in a fixed device array, and a chunk finds its gradient by binary search.
+// Chunks are numbered as the chunk list above orders them -- first every whole
+// chunk of the 16-byte aligned gradients, then everything else, each in tensor
+// order -- and fall to the same workgroups, so both passes add the same numbers
+// in the same order and return the same bits.
+// ---------------------------------------------------------------------------
+struct alignas(16) NormEntry {
+    uint64_t g;
+    uint64_t numel;
+    uint32_t first_whole;  // number of the gradient's first whole chunk among the whole chunks
+    uint32_t first_rest;   // number of its first other chunk among the other chunks
+    uint32_t n_whole;      // whole chunks it contributes to the first sequence
+    uint32_t dtype;
+};
+static_assert(sizeof(NormEntry) == 32, "NormEntry layout");
+
+// A slice of the table travels to the device array as a kernel argument (no copy engine, no
+// staging memory): at most kNormEntriesPerWrite entries per launch.
+constexpr uint32_t kNormEntriesPerWrite = 64;
+struct NormEntrySlice {
+    NormEntry e[kNormEntriesPerWrite];
+};
+__global__ __launch_bounds__(kNormEntriesPerWrite) void norm_table_write_kernel(NormEntry* __restrict__ table,
+                                                                                uint32_t first, uint32_t count,
+                                                                                const NormEntrySlice slice) {
+    if (threadIdx.x < count) table[first + threadIdx.x] = slice.e[threadIdx.x];
+}
+
+__global__ __launch_bounds__(kThreads) void grad_sumsq_table_kernel(const NormEntry* __restrict__ table, uint32_t n,
+                                                                    uint32_t total_whole, uint32_t n_chunks,
+                                                                    float inv_loss_scale,
+                                                                    double* __restrict__ partials) {
+    __shared__ float lds[kThreads / 64];
+    double total = 0.0;
+    for (uint32_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+        const bool whole = c < total_whole;
+        const uint32_t key = whole ? c : c - total_whole;
+        uint32_t lo = 0, hi = n;  // last entry whose first chunk number in this sequence is <= key
+        while (hi - lo > 1u) {
+            const uint32_t mid = (lo + hi) >> 1;
+            const uint32_t f = whole ? table[mid].first_whole : table[mid].first_rest;
+            if (f <= key) lo = mid; else hi = mid;
+        }
+        const NormEntry e = table[lo];
+        const uint32_t chunk = whole ? key - e.first_whole : e.n_whole + (key - e.first_rest);
+        const float acc = chunk_sumsq_dt((int)e.dtype, e.g, e.numel, chunk, inv_loss_scale);
+        const float bs = block_sum(acc, lds);
+        total += (double)bs;  // meaningful in thread 0 only
+    }
+    if (threadIdx.x == 0) partials[blockIdx.x] = total;
+}
+
 // Pass 2: one workgroup folds the partials in index order and derives the
 // clip coefficient with torch.nn.utils.clip_grad_norm_'s formula.
 __global__ __launch_bounds__(kThreads) void grad_norm_finish_kernel(const double* __restrict__ partials,
