@@ -261,6 +261,17 @@ int rt_stream_probe(rt_handle* h, void* p, const void* g, void* m, void* v, uint
 int rt_host_link_probe(rt_handle* h, uint64_t bytes, int reps, double out[3]);
 
 /*
+ * Device memory that is only held, not used: the state-placement search of the
+ * Python optimizer occupies memory with such blocks so that its next
+ * allocation lands further on in physical address order (see rt_stream_probe),
+ * without going through -- and leaving blocks behind in -- the caller's own
+ * caching allocator.  Nothing in the reference corresponds to it.
+ * rt_dev_hold returns RT_ENOMEM when the device has no such block left.
+ */
+int rt_dev_hold(rt_handle* h, uint64_t bytes, void** out);
+int rt_dev_release(rt_handle* h, void* p);
+
+/*
  * Self-test, nothing in the reference corresponds to it.  The update kernels
  * take the square root of the second moment (adamw.py:193) with a shortened
  * instruction sequence whenever a whole wavefront's values lie in

@@ -29,7 +29,7 @@ EXPORTS = (
     "rt_grad_norm", "rt_row_means", "rt_sr_copy", "rt_set_timing", "rt_last_kernel_ms", "rt_kernel_ms_history", "rt_streamed_stats",
     "rt_stream_probe", "rt_streamed_timeline", "rt_streamed_plan",
     "rt_step_streamed_async", "rt_streamed_wait", "rt_streamed_completed",
-    "rt_grad_norm_static", "rt_host_link_probe", "rt_selftest_sqrt",
+    "rt_grad_norm_static", "rt_host_link_probe", "rt_selftest_sqrt", "rt_dev_hold", "rt_dev_release",
 )
 
 
@@ -123,6 +123,10 @@ def lib() -> ctypes.CDLL:
     L.rt_grad_norm_static.argtypes = [vp, descs, u32, ctypes.c_float, ctypes.c_float, vp, vp]
     L.rt_host_link_probe.restype = i32
     L.rt_host_link_probe.argtypes = [vp, u64, i32, ctypes.POINTER(ctypes.c_double)]
+    L.rt_dev_hold.restype = i32
+    L.rt_dev_hold.argtypes = [vp, u64, ctypes.POINTER(vp)]
+    L.rt_dev_release.restype = i32
+    L.rt_dev_release.argtypes = [vp, vp]
     L.rt_selftest_sqrt.restype = i32
     L.rt_selftest_sqrt.argtypes = [vp, ctypes.POINTER(u64)]
     L.rt_row_means.restype = i32
@@ -240,6 +244,18 @@ class Handle:
         with self._lock:
             check(lib().rt_host_link_probe(self.ptr, int(nbytes), int(reps), out))
         return {"h2d_GBps": out[0], "d2h_GBps": out[1], "duplex_GBps_each_way": out[2]}
+
+    def dev_hold(self, nbytes: int) -> int:
+        """Address of a device block of ``nbytes`` that is only held (see rt_dev_hold); raises NativeError
+        with code RT_ENOMEM when there is none."""
+        out = ctypes.c_void_p()
+        with self._lock:
+            check(lib().rt_dev_hold(self.ptr, int(nbytes), ctypes.byref(out)))
+        return out.value
+
+    def dev_release(self, addr: int) -> None:
+        with self._lock:
+            check(lib().rt_dev_release(self.ptr, ctypes.c_void_p(addr)))
 
     def selftest_sqrt(self) -> int:
         """Number of floats in [2^-96, inf) on which the kernels' short sqrt differs from sqrtf (expected 0)."""

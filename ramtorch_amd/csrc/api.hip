@@ -134,6 +134,7 @@ struct rt_handle {
     DevBuf norm_partials;
     void* static_scratch = nullptr;       // this device's copy of `scratch`
     std::vector<NormEntry> norm_entries;  // host image of the table of rt_grad_norm_static
+    std::vector<NormEntry> norm_table;    // the same for rt_grad_norm
     std::vector<uint8_t> image;  // scratch for building a table image
     std::vector<DevTensor> tens;
     std::vector<uint32_t> ranges;       // first unit of each tensor of the fast kernel
@@ -299,7 +300,7 @@ struct Batch {            // tensors of one dtype combination inside a table ima
 
 struct Plan {
     size_t off_sets = 0, off_tensors = 0, off_ranges = 0, off_fast_tensors = 0, off_pieces = 0, off_chunks = 0,
-           off_gdt = 0, bytes = 0;
+           bytes = 0;
     uint32_t n_sets = 0, n_tensors = 0, n_chunks = 0;
     DevScalars first_set;   // passed by value when n_sets == 1
     std::vector<Batch> batches;
@@ -315,20 +316,17 @@ inline bool narrow_combo(uint32_t combo) {
     return true;
 }
 
-enum class ImageFor { Update, Norm };
-
 }  // namespace
 
 // Lays out [DevScalars sets][DevTensor records][first units][their DevTensor records][PieceRef pieces][ChunkRef list]
-// [g dtype bytes] in h->image.  Tensors are grouped by dtype combination so that each combination
+// in h->image.  Tensors are grouped by dtype combination so that each combination
 // is one contiguous range of every list = at most two launches.
-//   Update: whole fast units of plain tensors (16-byte aligned, no debug output, no centralization)
-//           become ranges; what such a tensor leaves over becomes pieces where the layout has a
-//           piece path (all arrays 16 bit, Philox noise), chunks of the generic kernel otherwise;
-//           every other tensor goes to the generic kernel chunk by chunk.
-//   Norm:   only the chunk list, over every element: whole chunks of aligned gradients first.
+// Whole fast units of plain tensors (16-byte aligned, no debug output, no centralization) become
+// ranges; what such a tensor leaves over becomes pieces where the layout has a piece path (all
+// arrays 16 bit, Philox noise), chunks of the generic kernel otherwise; every other tensor goes to
+// the generic kernel chunk by chunk.
 static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
-                        bool want_explicit, ImageFor what, Plan& plan) {
+                        bool want_explicit, Plan& plan) {
     // (scalars_idx, step) -> set index
     std::map<std::pair<uint32_t, uint32_t>, uint32_t> set_of;
     std::vector<DevScalars> sets;
@@ -393,27 +391,10 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
         b.combo = combo;
         b.first_range = (uint32_t)ranges.size();
         b.first_piece = (uint32_t)pieces.size();
-        const bool has_pieces = what == ImageFor::Update && !want_explicit && narrow_combo(combo);
+        const bool has_pieces = !want_explicit && narrow_combo(combo);
         auto plain = [&](const DevTensor& t) {
             return combo != kComboAny && (t.flags & kFlagAligned) && (t.dp | t.dm | t.dv | t.row_mean) == 0;
         };
-        if (what == ImageFor::Norm) {
-            // the chunk list only: whole chunks of aligned gradients first, then the rest
-            b.first_generic = (uint32_t)chunks.size();
-            for (size_t k = k0; k < k1; ++k) {
-                const uint32_t nw = plain(tens[k]) ? (uint32_t)(tens[k].numel / kChunkElems) : 0u;
-                for (uint32_t j = 0; j < nw; ++j) chunks.push_back(ChunkRef{(uint32_t)k, j});
-            }
-            for (size_t k = k0; k < k1; ++k) {
-                const uint32_t nw = plain(tens[k]) ? (uint32_t)(tens[k].numel / kChunkElems) : 0u;
-                const uint32_t nc = (uint32_t)((tens[k].numel + kChunkElems - 1) / kChunkElems);
-                for (uint32_t j = nw; j < nc; ++j) chunks.push_back(ChunkRef{(uint32_t)k, j});
-            }
-            b.n_generic = (uint32_t)chunks.size() - b.first_generic;
-            plan.batches.push_back(b);
-            k0 = k1;
-            continue;
-        }
         uint32_t units = 0;
         for (size_t k = k0; k < k1; ++k) {
             const DevTensor& t = tens[k];
@@ -465,8 +446,7 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
     plan.off_fast_tensors = plan.off_ranges + align_up(ranges.size() * sizeof(uint32_t), 128);
     plan.off_pieces = plan.off_fast_tensors + align_up(fast_tens.size() * sizeof(DevTensor), 128);
     plan.off_chunks = plan.off_pieces + align_up(pieces.size() * sizeof(PieceRef), 128);
-    plan.off_gdt = plan.off_chunks + align_up(chunks.size() * sizeof(ChunkRef), 128);
-    plan.bytes = plan.off_gdt + (what == ImageFor::Norm ? align_up(tens.size(), 128) : 0);
+    plan.bytes = plan.off_chunks + align_up(chunks.size() * sizeof(ChunkRef), 128);
     h->image.assign(plan.bytes, 0);
     uint8_t* img = h->image.data();
     if (!sets.empty()) memcpy(img + plan.off_sets, sets.data(), sets.size() * sizeof(DevScalars));
@@ -476,8 +456,6 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
         memcpy(img + plan.off_fast_tensors, fast_tens.data(), fast_tens.size() * sizeof(DevTensor));
     if (!pieces.empty()) memcpy(img + plan.off_pieces, pieces.data(), pieces.size() * sizeof(PieceRef));
     if (!chunks.empty()) memcpy(img + plan.off_chunks, chunks.data(), chunks.size() * sizeof(ChunkRef));
-    if (what == ImageFor::Norm)
-        for (size_t k = 0; k < order.size(); ++k) img[plan.off_gdt + k] = descs[order[k]].g_dtype;
 }
 
 // Puts h->image into a free table slot (skipping the copy when the slot's
@@ -572,7 +550,7 @@ static int launch_update(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, 
                          uint64_t seed, int noise_mode, const float* d_clip_coef, const uint32_t* d_skip,
                          hipStream_t stream) {
     Plan plan;
-    build_image(h, descs, n, scalars, noise_mode == RT_NOISE_EXPLICIT, ImageFor::Update, plan);
+    build_image(h, descs, n, scalars, noise_mode == RT_NOISE_EXPLICIT, plan);
     if (plan.n_tensors == 0) return RT_OK;
     TableSlot* slot = nullptr;
     int rc = stage_image(h, plan, stream, &slot);
@@ -738,6 +716,43 @@ int rt_step_multi(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const r
     return launch_update(h, descs, n, scalars, seed, noise_mode, d_clip_coef, d_skip, (hipStream_t)stream);
 }
 
+// The gradient table of the norm pass: one NormEntry per non-empty gradient.  Chunks of 8192
+// elements are numbered in two sequences -- every whole chunk of the 16-byte aligned gradients
+// first, then all other chunks, each in tensor order -- and chunk c belongs to workgroup c mod grid.
+static int build_norm_table(const rt_tensor_desc* descs, uint32_t n, size_t max_entries, std::vector<NormEntry>& tab,
+                            uint64_t& n_whole, uint64_t& n_rest) {
+    tab.clear();
+    n_whole = n_rest = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        const rt_tensor_desc& d = descs[i];
+        if (d.g_dtype > RT_DT_F16) return fail(RT_EINVAL, "tensor %u: g_dtype %d unknown", i, d.g_dtype);
+        if (d.host_mask) return fail(RT_EINVAL, "tensor %u: host_mask set (grads must be device resident)", i);
+        if (d.numel == 0) continue;
+        if (!d.g) return fail(RT_EINVAL, "tensor %u: g is NULL", i);
+        if ((uintptr_t)d.g % dtype_size(d.g_dtype))
+            return fail(RT_EINVAL, "tensor %u: g not aligned to its element size", i);
+        if (d.numel / kChunkElems >= 0xFFFFFFFFull) return fail(RT_EUNSUPPORTED, "tensor %u: numel too large", i);
+        if (tab.size() >= max_entries)
+            return fail(RT_EUNSUPPORTED,
+                        "rt_grad_norm_static takes at most %zu non-empty gradients per call (its table is a fixed "
+                        "device array); use rt_grad_norm", max_entries);
+        const uint64_t chunks = (d.numel + kChunkElems - 1) / kChunkElems;
+        const uint64_t whole = ((uintptr_t)d.g & 15u) == 0 ? d.numel / kChunkElems : 0;
+        NormEntry e;
+        e.g = (uint64_t)d.g;
+        e.numel = d.numel;
+        e.first_whole = (uint32_t)n_whole;
+        e.first_rest = (uint32_t)n_rest;
+        e.n_whole = (uint32_t)whole;
+        e.dtype = d.g_dtype;
+        tab.push_back(e);
+        n_whole += whole;
+        n_rest += chunks - whole;
+        if (n_whole + n_rest > kMaxGrid) return fail(RT_EUNSUPPORTED, "too many elements in one call");
+    }
+    return RT_OK;
+}
+
 int rt_grad_norm(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, float inv_loss_scale, float max_norm,
                  void* d_out, void* stream_) {
     if (!h) return fail(RT_EINVAL, "handle is NULL");
@@ -745,54 +760,27 @@ int rt_grad_norm(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, float in
     if (n > 0 && !descs) return fail(RT_EINVAL, "descs is NULL");
     hipStream_t stream = (hipStream_t)stream_;
     HIP_TRY(hipSetDevice(h->device));
-    // Reuse the table builder with a descriptor copy that only carries g.
-    std::vector<rt_tensor_desc> gd(descs, descs + n);
-    rt_scalars one;
-    memset(&one, 0, sizeof(one));
-    one.inv_loss_scale = 1.0f;
-    uint64_t total_chunks = 0;
-    for (uint32_t i = 0; i < n; ++i) {
-        rt_tensor_desc& d = gd[i];
-        if (d.g_dtype > RT_DT_F16) return fail(RT_EINVAL, "tensor %u: g_dtype %d unknown", i, d.g_dtype);
-        if (d.numel && !d.g) return fail(RT_EINVAL, "tensor %u: g is NULL", i);
-        if (d.numel && ((uintptr_t)d.g % dtype_size(d.g_dtype)))
-            return fail(RT_EINVAL, "tensor %u: g not aligned to its element size", i);
-        if (d.numel / kChunkElems >= 0xFFFFFFFFull) return fail(RT_EUNSUPPORTED, "tensor %u: numel too large", i);
-        total_chunks += (d.numel + kChunkElems - 1) / kChunkElems;
-        if (total_chunks > kMaxGrid) return fail(RT_EUNSUPPORTED, "too many elements in one call");
-        if (d.host_mask) return fail(RT_EINVAL, "tensor %u: host_mask set (grads must be device resident)", i);
-        d.p = d.m = d.v = nullptr;
-        d.noise_p = d.noise_m = d.noise_v = nullptr;
-        d.dbg_p = d.dbg_m = d.dbg_v = nullptr;
-        d.row_mean = nullptr;
-        d.scalars_idx = 0;
-        d.step = 0;
-        d.elem_offset = 0;
-        // one dtype combination => one chunk list; the real gradient dtype is looked up per tensor
-        d.p_dtype = d.g_dtype = d.m_dtype = d.v_dtype = RT_DT_BF16;
-    }
-    Plan plan;
-    build_image(h, gd.data(), n, &one, false, ImageFor::Norm, plan);
-    {
-        // build_image keeps the input order inside one combination
-        uint8_t* gdt = h->image.data() + plan.off_gdt;
-        uint32_t k = 0;
-        for (uint32_t i = 0; i < n; ++i)
-            if (descs[i].numel != 0) gdt[k++] = descs[i].g_dtype;
-    }
-    int rc = dev_reserve(h->norm_partials, kNormPartials * sizeof(double));
+    std::vector<NormEntry>& tab = h->norm_table;
+    uint64_t n_whole = 0, n_rest = 0;
+    int rc = build_norm_table(descs, n, SIZE_MAX, tab, n_whole, n_rest);
+    if (rc != RT_OK) return rc;
+    rc = dev_reserve(h->norm_partials, kNormPartials * sizeof(double));
     if (rc != RT_OK) return rc;
     // With nothing to sum the finish kernel reads no partials (a total of zero).  (2048 - 4096
-    // workgroups walking the chunk list read at 6.9 - 7.0 TB/s; more workgroups were slower.)
-    const uint32_t grid = std::min<uint32_t>(kNormPartials, plan.n_chunks);
-    if (plan.n_chunks != 0) {
+    // workgroups read at 6.6 - 7.0 TB/s; more workgroups were slower.)
+    const uint32_t n_chunks = (uint32_t)(n_whole + n_rest);
+    const uint32_t grid = std::min<uint32_t>(kNormPartials, n_chunks);
+    if (n_chunks != 0) {
+        // the table goes through a staging slot: the same gradients step after step upload nothing
+        Plan plan;
+        plan.bytes = tab.size() * sizeof(NormEntry);
+        h->image.assign((const uint8_t*)tab.data(), (const uint8_t*)tab.data() + plan.bytes);
         TableSlot* slot = nullptr;
         rc = stage_image(h, plan, stream, &slot);
         if (rc != RT_OK) return rc;
-        const uint8_t* base = (const uint8_t*)slot->dev.ptr;
-        hipLaunchKernelGGL(grad_sumsq_kernel, dim3(grid), dim3(kThreads), 0, stream,
-                           (const DevTensor*)(base + plan.off_tensors), (const ChunkRef*)(base + plan.off_chunks),
-                           plan.n_chunks, base + plan.off_gdt, inv_loss_scale, (double*)h->norm_partials.ptr);
+        hipLaunchKernelGGL(grad_sumsq_table_kernel, dim3(grid), dim3(kThreads), 0, stream,
+                           (const NormEntry*)slot->dev.ptr, (uint32_t)tab.size(), (uint32_t)n_whole, n_chunks,
+                           inv_loss_scale, (double*)h->norm_partials.ptr);
         HIP_TRY(hipGetLastError());
         HIP_TRY(hipEventRecord(slot->done, stream));
         slot->in_flight = true;
@@ -811,38 +799,10 @@ int rt_grad_norm_static(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, f
     if (!h->static_scratch) return fail(RT_EHIP, "the static scratch array has no address on device %d", h->device);
     hipStream_t stream = (hipStream_t)stream_;
     HIP_TRY(hipSetDevice(h->device));
-    // Chunks are numbered as the chunk list of rt_grad_norm orders them: every whole chunk of the
-    // 16-byte aligned gradients first, then all other chunks, each in tensor order.
     std::vector<NormEntry>& tab = h->norm_entries;  // capacity reserved by rt_create
-    tab.clear();
     uint64_t n_whole = 0, n_rest = 0;
-    for (uint32_t i = 0; i < n; ++i) {
-        const rt_tensor_desc& d = descs[i];
-        if (d.g_dtype > RT_DT_F16) return fail(RT_EINVAL, "tensor %u: g_dtype %d unknown", i, d.g_dtype);
-        if (d.host_mask) return fail(RT_EINVAL, "tensor %u: host_mask set (grads must be device resident)", i);
-        if (d.numel == 0) continue;
-        if (!d.g) return fail(RT_EINVAL, "tensor %u: g is NULL", i);
-        if ((uintptr_t)d.g % dtype_size(d.g_dtype))
-            return fail(RT_EINVAL, "tensor %u: g not aligned to its element size", i);
-        if (d.numel / kChunkElems >= 0xFFFFFFFFull) return fail(RT_EUNSUPPORTED, "tensor %u: numel too large", i);
-        if (tab.size() >= kStaticMaxTensors)
-            return fail(RT_EUNSUPPORTED,
-                        "rt_grad_norm_static takes at most %u non-empty gradients per call (its table is a fixed "
-                        "device array); use rt_grad_norm", kStaticMaxTensors);
-        const uint64_t chunks = (d.numel + kChunkElems - 1) / kChunkElems;
-        const uint64_t whole = ((uintptr_t)d.g & 15u) == 0 ? d.numel / kChunkElems : 0;
-        NormEntry e;
-        e.g = (uint64_t)d.g;
-        e.numel = d.numel;
-        e.first_whole = (uint32_t)n_whole;
-        e.first_rest = (uint32_t)n_rest;
-        e.n_whole = (uint32_t)whole;
-        e.dtype = d.g_dtype;
-        tab.push_back(e);
-        n_whole += whole;
-        n_rest += chunks - whole;
-        if (n_whole + n_rest > kMaxGrid) return fail(RT_EUNSUPPORTED, "too many elements in one call");
-    }
+    const int rc = build_norm_table(descs, n, kStaticMaxTensors, tab, n_whole, n_rest);
+    if (rc != RT_OK) return rc;
     double* partials = (double*)h->static_scratch;
     NormEntry* table = (NormEntry*)((uint8_t*)h->static_scratch + kStaticPartialsBytes);
     const uint32_t n_chunks = (uint32_t)(n_whole + n_rest);
@@ -1148,7 +1108,7 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
             pieces[c].push_back(q);
         }
         build_image(h, pieces[c].data(), (uint32_t)pieces[c].size(), scalars, noise_mode == RT_NOISE_EXPLICIT,
-                    ImageFor::Update, plans[c]);
+                    plans[c]);
         plan_off[c] = align_up(blob.size(), 256);
         blob.resize(plan_off[c] + plans[c].bytes);
         if (plans[c].bytes) memcpy(blob.data() + plan_off[c], h->image.data(), plans[c].bytes);
@@ -1439,6 +1399,29 @@ int rt_host_link_probe(rt_handle* h, uint64_t bytes, int reps, double out[3]) {
     out[2] = total / run(true, true);
     release();
     HIP_TRY(hipGetLastError());
+    return RT_OK;
+}
+
+int rt_dev_hold(rt_handle* h, uint64_t bytes, void** out) {
+    if (!h || !out) return fail(RT_EINVAL, "NULL argument");
+    *out = nullptr;
+    if (bytes == 0) return fail(RT_EINVAL, "bytes must be positive");
+    HIP_TRY(hipSetDevice(h->device));
+    void* p = nullptr;
+    const hipError_t e = hipMalloc(&p, bytes);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();  // a failed allocation must not surface again behind a later launch
+        return fail(RT_ENOMEM, "hipMalloc(%llu) failed: %s", (unsigned long long)bytes, hipGetErrorString(e));
+    }
+    *out = p;
+    return RT_OK;
+}
+
+int rt_dev_release(rt_handle* h, void* p) {
+    if (!h) return fail(RT_EINVAL, "handle is NULL");
+    if (!p) return RT_OK;
+    HIP_TRY(hipSetDevice(h->device));
+    HIP_TRY(hipFree(p));
     return RT_OK;
 }
 

@@ -1067,32 +1067,14 @@ __device__ __forceinline__ float chunk_sumsq_dt(int dt, uint64_t g_addr, uint64_
     return chunk_sumsq<RT_DT_F16>(g_addr, n, chunk, inv_loss_scale);
 }
 
-// Pass 1 of the global grad norm: workgroup b accumulates the chunks
-// b, b + gridDim.x, ... and writes one partial sum of squares.
-__global__ __launch_bounds__(kThreads) void grad_sumsq_kernel(const DevTensor* __restrict__ tensors,
-                                                              const ChunkRef* __restrict__ chunks,
-                                                              uint32_t n_chunks, const uint8_t* __restrict__ gdt,
-                                                              float inv_loss_scale, double* __restrict__ partials) {
-    __shared__ float lds[kThreads / 64];
-    double total = 0.0;
-    for (uint32_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-        const ChunkRef cr = chunks[c];
-        const DevTensor& t = tensors[cr.tensor];
-        const float acc = chunk_sumsq_dt(gdt[cr.tensor], t.g, t.numel, cr.chunk, inv_loss_scale);
-        const float bs = block_sum(acc, lds);
-        total += (double)bs;  // meaningful in thread 0 only
-    }
-    if (threadIdx.x == 0) partials[blockIdx.x] = total;
-}
-
 // ---------------------------------------------------------------------------
-// The same pass without a chunk list, for the entry point that allocates
-// nothing: the only table is one NormEntry per gradient, small enough to live
-// in a fixed device array, and a chunk finds its gradient by binary search.
-// Chunks are numbered as the chunk list above orders them -- first every whole
+// Pass 1 of the global grad norm: workgroup b accumulates the chunks
+// b, b + gridDim.x, ... and writes one partial sum of squares.  The only table
+// is one NormEntry per gradient (small enough to live in a fixed device array
+// for the entry point that allocates nothing); a chunk finds its gradient by
+// binary search.  Chunks are numbered in two sequences -- first every whole
 // chunk of the 16-byte aligned gradients, then everything else, each in tensor
-// order -- and fall to the same workgroups, so both passes add the same numbers
-// in the same order and return the same bits.
+// order -- so that most workgroups see nothing but whole chunks.
 // ---------------------------------------------------------------------------
 struct alignas(16) NormEntry {
     uint64_t g;

@@ -115,6 +115,9 @@ class AdamW(Optimizer):
             pool and all ``ema_squared`` tensors out of another and places the two pools in
             different HBM regions, found by measurement at construction (see
             ``ramtorch_amd/placement.py``; the outcome is in ``state_placement_report``).
+            While it searches, the constructor occupies up to half of the free device memory
+            (at most 112 GiB, for at most 8 s) through the library and gives all of it back;
+            torch's caching allocator only ever sees the two pools.
             "plain" allocates every state tensor on its own, as the reference does.
     """
 

@@ -3,6 +3,7 @@ against the reference's own op sequence, unbiasedness of the Philox rounding,
 grad-norm clip, centralization, copy_stochastic_.  Run with ``-m gpu``.
 """
 import copy
+import time
 
 import numpy as np
 import pytest
@@ -657,3 +658,46 @@ def test_zeros_denormals_and_tiny_second_moments_take_the_full_sqrt():
         got, want = t.cpu().numpy().view(np.uint32), a.view(np.uint32)
         both_nan = np.isnan(t.cpu().numpy()) & np.isnan(a)
         assert ((got == want) | both_nan).all(), name
+
+
+def test_state_placement_with_most_of_hbm_occupied_falls_back_quietly():
+    """The constructor's placement search occupies memory only through the library and only a bounded
+    share of what is free: with most of HBM taken it ends at once, leaves torch's caching allocator
+    alone, and the optimizer steps exactly like one with plainly allocated states."""
+    GIB = 1 << 30
+    torch.cuda.empty_cache()
+    free, _ = torch.cuda.mem_get_info()
+    hog = [torch.empty(8 * GIB, dtype=torch.uint8, device="cuda") for _ in range(int((free - 16 * GIB) // (8 * GIB)))]
+    try:
+        n = 1 << 29   # 1 GiB of bf16 per array: the smallest set the search is used for
+        gen = torch.Generator("cuda").manual_seed(5)
+        base = (torch.randn(n, device="cuda", generator=gen) * 0.02).bfloat16()
+        grad = (torch.randn(n, device="cuda", generator=gen) * 1e-3).bfloat16()
+        p1 = torch.nn.Parameter(base.clone(), requires_grad=False)
+        p2 = torch.nn.Parameter(base.clone(), requires_grad=False)
+        del base
+        torch.cuda.synchronize()
+        reserved0 = torch.cuda.memory_reserved()
+        t0 = time.monotonic()
+        opt1 = ramtorch_amd.AdamW([p1], storage_device="cuda", seed=3, state_placement="auto", **HP0)
+        took = time.monotonic() - t0
+        rep = opt1.state_placement_report
+        assert rep is not None and rep["tries"] >= 1 and isinstance(rep["placed"], bool), rep
+        assert took < 10.0, took
+        # torch holds the two pools and nothing else that it did not hold before
+        assert torch.cuda.memory_reserved() - reserved0 <= 2 * GIB + (64 << 20)
+        st = opt1.state[p1]
+        assert float(st["ema"].float().abs().max()) == 0.0 and float(st["ema_squared"].float().abs().max()) == 0.0
+        opt2 = ramtorch_amd.AdamW([p2], storage_device="cuda", seed=3, state_placement="plain", **HP0)
+        for _ in range(2):
+            p1.grad = grad
+            p2.grad = grad
+            opt1.step()
+            opt2.step()
+        torch.cuda.synchronize()
+        assert torch.equal(p1.view(torch.int16), p2.view(torch.int16))
+        for k in ("ema", "ema_squared"):
+            assert torch.equal(opt1.state[p1][k].view(torch.int16), opt2.state[p2][k].view(torch.int16))
+    finally:
+        del hog
+        torch.cuda.empty_cache()
