@@ -85,7 +85,7 @@ def build_gather(verbose: bool = False) -> str:
            "-I" + sysconfig.get_paths()["include"]]
     cmd += ["-I" + i for i in cpp_extension.include_paths()]
     cmd += [GATHER_SRC, "-o", gather_path(), "-L" + torch_lib, "-ltorch_python", "-ltorch", "-ltorch_cpu", "-lc10",
-            "-Wl,-rpath," + torch_lib]
+            "-Wl,-rpath," + torch_lib, "-pthread"]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)

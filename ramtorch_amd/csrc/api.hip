@@ -6,6 +6,7 @@
 #include <algorithm>
 #include <chrono>
 #include <cstdarg>
+#include <cstddef>
 #include <cstdio>
 #include <cstdlib>
 #include <climits>
@@ -66,6 +67,7 @@ struct TableSlot {
     void* host = nullptr;  // pinned; keeps the image last uploaded to `dev`
     size_t host_cap = 0;
     size_t valid_bytes = 0;  // bytes of `host` that `dev` currently mirrors
+    uint64_t static_gen = 0; // layout generation of the lists behind the scalars, 0 = unknown
     hipEvent_t done = nullptr;
     bool in_flight = false;
 };
@@ -111,6 +113,39 @@ struct Streamed {
 }  // namespace
 
 // ---------------------------------------------------------------------------
+// what one table image holds
+// ---------------------------------------------------------------------------
+namespace {
+
+struct Batch {            // tensors of one dtype combination inside a table image
+    uint32_t combo;
+    uint32_t first_range, n_ranges, n_units;   // fast kernel: entries of the range list, fast units
+    uint32_t first_piece, n_pieces;            // pieces served by the fast kernel's first workgroups
+    uint32_t first_generic, n_generic;         // chunk range of the generic kernel
+};
+
+struct Plan {
+    size_t off_sets = 0, off_tensors = 0, off_ranges = 0, off_fast_tensors = 0, off_pieces = 0, off_chunks = 0,
+           bytes = 0;
+    uint32_t n_sets = 0, n_tensors = 0, n_chunks = 0;
+    DevScalars first_set;   // passed by value when n_sets == 1
+    std::vector<Batch> batches;
+    std::vector<std::pair<uint32_t, uint32_t>> set_keys;  // set index -> (scalars_idx, step)
+};
+
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// All arrays 16 bit wide: the layouts whose fast kernel has a piece path.
+inline bool narrow_combo(uint32_t combo) {
+    if (combo & 0x100u) return false;
+    for (int k = 0; k < 4; ++k)
+        if (((combo >> (2 * k)) & 3u) == RT_DT_F32) return false;
+    return true;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
 // Device memory of the entry point that allocates nothing (rt_grad_norm_static): the per-workgroup
 // partial sums and the gradient table, in one array that is part of the loaded code object -- every
 // GPU the library runs on holds its own copy at its own address until the process ends.  Host code
@@ -135,6 +170,19 @@ struct rt_handle {
     void* static_scratch = nullptr;       // this device's copy of `scratch`
     std::vector<NormEntry> norm_entries;  // host image of the table of rt_grad_norm_static
     std::vector<NormEntry> norm_table;    // the same for rt_grad_norm
+    // The table image of the most recent rt_step_multi call, kept so that a call over the same tensors
+    // (same addresses, sizes, types; every step count advanced by one common amount) rebuilds only
+    // the per-step scalars.
+    struct LayoutCache {
+        bool valid = false;
+        int noise_mode = 0;
+        uint64_t gen = 0;
+        std::vector<rt_tensor_desc> descs;
+        std::vector<uint8_t> image;
+        std::vector<uint8_t> cen;  // per set: centralization was on when the image was built
+        Plan plan;
+    } layout;
+    uint64_t layout_gen = 0;
     std::vector<uint8_t> image;  // scratch for building a table image
     std::vector<DevTensor> tens;
     std::vector<uint32_t> ranges;       // first unit of each tensor of the fast kernel
@@ -289,34 +337,6 @@ static int validate(const rt_tensor_desc* descs, uint32_t n, const rt_scalars* s
 // ---------------------------------------------------------------------------
 // table building and launch
 // ---------------------------------------------------------------------------
-namespace {
-
-struct Batch {            // tensors of one dtype combination inside a table image
-    uint32_t combo;
-    uint32_t first_range, n_ranges, n_units;   // fast kernel: entries of the range list, fast units
-    uint32_t first_piece, n_pieces;            // pieces served by the fast kernel's first workgroups
-    uint32_t first_generic, n_generic;         // chunk range of the generic kernel
-};
-
-struct Plan {
-    size_t off_sets = 0, off_tensors = 0, off_ranges = 0, off_fast_tensors = 0, off_pieces = 0, off_chunks = 0,
-           bytes = 0;
-    uint32_t n_sets = 0, n_tensors = 0, n_chunks = 0;
-    DevScalars first_set;   // passed by value when n_sets == 1
-    std::vector<Batch> batches;
-};
-
-inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
-
-// All arrays 16 bit wide: the layouts whose fast kernel has a piece path.
-inline bool narrow_combo(uint32_t combo) {
-    if (combo & 0x100u) return false;
-    for (int k = 0; k < 4; ++k)
-        if (((combo >> (2 * k)) & 3u) == RT_DT_F32) return false;
-    return true;
-}
-
-}  // namespace
 
 // Lays out [DevScalars sets][DevTensor records][first units][their DevTensor records][PieceRef pieces][ChunkRef list]
 // in h->image.  Tensors are grouped by dtype combination so that each combination
@@ -436,6 +456,8 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
         k0 = k1;
     }
 
+    plan.set_keys.assign(sets.size(), {0u, 0u});
+    for (const auto& kv : set_of) plan.set_keys[kv.second] = kv.first;
     plan.n_sets = (uint32_t)sets.size();
     plan.n_tensors = (uint32_t)tens.size();
     plan.n_chunks = (uint32_t)chunks.size();
@@ -458,9 +480,11 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
     if (!chunks.empty()) memcpy(img + plan.off_chunks, chunks.data(), chunks.size() * sizeof(ChunkRef));
 }
 
-// Puts h->image into a free table slot (skipping the copy when the slot's
-// device memory already holds the same bytes) and returns the slot.
-static int stage_image(rt_handle* h, const Plan& plan, hipStream_t stream, TableSlot** out) {
+// Puts a table image into a free table slot (skipping what the slot's device memory already
+// holds) and returns the slot.  `static_gen` != 0 names the layout the lists behind the scalars
+// belong to: a slot that holds the same generation is not even compared.
+static int stage_image(rt_handle* h, const Plan& plan, const uint8_t* img, uint64_t static_gen, hipStream_t stream,
+                       TableSlot** out) {
     TableSlot& s = h->slots[h->slot_counter++ % kSlots];
     if (s.in_flight) {
         HIP_TRY(hipEventSynchronize(s.done));
@@ -484,18 +508,20 @@ static int stage_image(rt_handle* h, const Plan& plan, hipStream_t stream, Table
     // Two regions: the DevScalars sets change with every step, the lists behind them only when the
     // tensors do; each region is copied only if the device copy differs.
     const size_t split = std::min(plan.off_tensors, plan.bytes);
-    const uint8_t* img = h->image.data();
     const bool known = s.valid_bytes == plan.bytes;
     if (split > 0 && !(known && memcmp(s.host, img, split) == 0)) {
         memcpy(s.host, img, split);
         HIP_TRY(hipMemcpyAsync(s.dev.ptr, s.host, split, hipMemcpyHostToDevice, stream));
     }
-    if (plan.bytes > split && !(known && memcmp((uint8_t*)s.host + split, img + split, plan.bytes - split) == 0)) {
+    const bool same_gen = known && static_gen != 0 && s.static_gen == static_gen;
+    if (plan.bytes > split && !same_gen &&
+        !(known && memcmp((uint8_t*)s.host + split, img + split, plan.bytes - split) == 0)) {
         memcpy((uint8_t*)s.host + split, img + split, plan.bytes - split);
         HIP_TRY(hipMemcpyAsync((uint8_t*)s.dev.ptr + split, (uint8_t*)s.host + split, plan.bytes - split,
                                hipMemcpyHostToDevice, stream));
     }
     s.valid_bytes = plan.bytes;
+    s.static_gen = static_gen;
     *out = &s;
     return RT_OK;
 }
@@ -546,14 +572,63 @@ static int enqueue_kernels(const Plan& plan, const uint8_t* base, uint64_t seed,
     return RT_OK;
 }
 
+// Whether `descs` describe the tensors of the cached layout: everything but the step counts equal,
+// and every step count ahead of the cached one by the same amount (*delta).
+static bool same_layout(const rt_handle::LayoutCache& lc, const rt_tensor_desc* descs, uint32_t n, int noise_mode,
+                        const rt_scalars* scalars, uint32_t n_scalars, uint32_t* delta) {
+    if (!lc.valid || lc.noise_mode != noise_mode || lc.descs.size() != n || n == 0) return false;
+    static_assert(offsetof(rt_tensor_desc, step) == 116 && sizeof(rt_tensor_desc) == 136, "rt_tensor_desc layout");
+    const uint32_t d0 = descs[0].step - lc.descs[0].step;
+    for (uint32_t i = 0; i < n; ++i) {
+        const uint8_t* a = (const uint8_t*)&descs[i];
+        const uint8_t* b = (const uint8_t*)&lc.descs[i];
+        if (memcmp(a, b, 116) != 0 || memcmp(a + 120, b + 120, 16) != 0) return false;
+        if (descs[i].step - lc.descs[i].step != d0) return false;
+    }
+    for (size_t j = 0; j < lc.plan.set_keys.size(); ++j) {
+        const uint32_t si = lc.plan.set_keys[j].first;
+        if (si >= n_scalars || (scalars[si].centralization != 0.0f) != (lc.cen[j] != 0)) return false;
+    }
+    *delta = d0;
+    return true;
+}
+
 static int launch_update(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
-                         uint64_t seed, int noise_mode, const float* d_clip_coef, const uint32_t* d_skip,
-                         hipStream_t stream) {
-    Plan plan;
-    build_image(h, descs, n, scalars, noise_mode == RT_NOISE_EXPLICIT, plan);
+                         uint32_t n_scalars, uint64_t seed, int noise_mode, const float* d_clip_coef,
+                         const uint32_t* d_skip, hipStream_t stream) {
+    rt_handle::LayoutCache& lc = h->layout;
+    uint32_t delta = 0;
+    if (same_layout(lc, descs, n, noise_mode, scalars, n_scalars, &delta)) {
+        // only the per-step scalars are new: the arguments were validated when the layout was built
+        DevScalars* sets = (DevScalars*)(lc.image.data() + lc.plan.off_sets);
+        for (size_t j = 0; j < lc.plan.set_keys.size(); ++j) {
+            auto& key = lc.plan.set_keys[j];
+            key.second += delta;
+            memset(&sets[j], 0, sizeof(DevScalars));
+            sets[j].s = scalars[key.first];
+            sets[j].step = key.second;
+        }
+        if (!lc.plan.set_keys.empty()) lc.plan.first_set = sets[0];
+        if (delta != 0)
+            for (uint32_t i = 0; i < n; ++i) lc.descs[i].step = descs[i].step;
+    } else {
+        lc.valid = false;
+        int rc = validate(descs, n, scalars, n_scalars, noise_mode, /*allow_host=*/false);
+        if (rc != RT_OK) return rc;
+        build_image(h, descs, n, scalars, noise_mode == RT_NOISE_EXPLICIT, lc.plan);
+        lc.image = h->image;
+        lc.descs.assign(descs, descs + n);
+        lc.cen.resize(lc.plan.set_keys.size());
+        for (size_t j = 0; j < lc.plan.set_keys.size(); ++j)
+            lc.cen[j] = scalars[lc.plan.set_keys[j].first].centralization != 0.0f;
+        lc.noise_mode = noise_mode;
+        lc.gen = ++h->layout_gen;
+        lc.valid = true;
+    }
+    const Plan& plan = lc.plan;
     if (plan.n_tensors == 0) return RT_OK;
     TableSlot* slot = nullptr;
-    int rc = stage_image(h, plan, stream, &slot);
+    int rc = stage_image(h, plan, lc.image.data(), lc.gen, stream, &slot);
     if (rc != RT_OK) return rc;
     std::pair<hipEvent_t, hipEvent_t>* tp = nullptr;
     if (h->timing) {
@@ -709,11 +784,11 @@ int rt_step_multi(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const r
                   uint32_t n_scalars, uint64_t seed, int noise_mode, const float* d_clip_coef,
                   const uint32_t* d_skip, void* stream) {
     if (!h) return fail(RT_EINVAL, "handle is NULL");
-    int rc = validate(descs, n, scalars, n_scalars, noise_mode, /*allow_host=*/false);
-    if (rc != RT_OK) return rc;
-    if (n == 0) return RT_OK;
+    if (n == 0) return validate(descs, n, scalars, n_scalars, noise_mode, /*allow_host=*/false);
+    if (!descs || !scalars || n_scalars == 0 || (noise_mode != RT_NOISE_PHILOX && noise_mode != RT_NOISE_EXPLICIT))
+        return validate(descs, n, scalars, n_scalars, noise_mode, /*allow_host=*/false);  // names the bad argument
     HIP_TRY(hipSetDevice(h->device));
-    return launch_update(h, descs, n, scalars, seed, noise_mode, d_clip_coef, d_skip, (hipStream_t)stream);
+    return launch_update(h, descs, n, scalars, n_scalars, seed, noise_mode, d_clip_coef, d_skip, (hipStream_t)stream);
 }
 
 // The gradient table of the norm pass: one NormEntry per non-empty gradient.  Chunks of 8192
@@ -776,7 +851,7 @@ int rt_grad_norm(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, float in
         plan.bytes = tab.size() * sizeof(NormEntry);
         h->image.assign((const uint8_t*)tab.data(), (const uint8_t*)tab.data() + plan.bytes);
         TableSlot* slot = nullptr;
-        rc = stage_image(h, plan, stream, &slot);
+        rc = stage_image(h, plan, h->image.data(), 0, stream, &slot);
         if (rc != RT_OK) return rc;
         hipLaunchKernelGGL(grad_sumsq_table_kernel, dim3(grid), dim3(kThreads), 0, stream,
                            (const NormEntry*)slot->dev.ptr, (uint32_t)tab.size(), (uint32_t)n_whole, n_chunks,

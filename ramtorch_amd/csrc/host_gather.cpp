@@ -17,6 +17,7 @@
 #include <cstdint>
 #include <algorithm>
 #include <cstring>
+#include <thread>
 #include <vector>
 
 #include "../../include/ramtorch_sr_adamw.h"
@@ -256,6 +257,98 @@ PyObject* gather_group(PyObject*, PyObject* const* args, Py_ssize_t nargs) {
     return out;
 }
 
+// verify_layout(params, expect_addr, n) -> bool
+// The cheap per-step check of a frozen layout: params is the flat list of parameters the layout was
+// recorded for, expect_addr the address of n triples of uint64 (data pointer of the parameter, data
+// pointer of its gradient or 0 for "no gradient", RT_DT_* code of the gradient).  True when every
+// parameter is still an exact Tensor / Parameter at the recorded address whose gradient is where it
+// was (or still absent), dense, contiguous, of the recorded dtype and of the parameter's size.
+// Reads what gather_group reads of a parameter and its gradient, with the same software prefetch,
+// and nothing of the states; it changes nothing.
+// One contiguous range of the check.  Only reads: object headers, tensor records, storages.
+bool verify_range(PyObject* params, const uint64_t* expect, Py_ssize_t lo, Py_ssize_t hi) {
+    constexpr Py_ssize_t kAhead = 8;
+    constexpr Py_ssize_t kSlots = 4 * kAhead;
+    const c10::TensorImpl* pimpl[kSlots] = {};
+    auto stage = [&](int level, Py_ssize_t i) {
+        if (i < lo || i >= hi) return;
+        const Py_ssize_t r = i % kSlots;
+        PyObject* po = PyList_GET_ITEM(params, i);
+        switch (level) {
+            case 0: touch(po); break;
+            case 1:
+                pimpl[r] = exact_tensor(po) ? THPVariable_Unpack(po).unsafeGetTensorImpl() : nullptr;
+                if (pimpl[r]) touch(pimpl[r], 4);
+                break;
+            case 2:
+                if (pimpl[r]) {
+                    touch(pimpl[r]->autograd_meta(), 2);
+                    touch(pimpl[r]->unsafe_storage().unsafeGetStorageImpl());
+                }
+                break;
+            default:
+                if (pimpl[r]) {
+                    const at::Tensor& g = THPVariable_Unpack(po).grad();
+                    if (g.defined()) touch(g.unsafeGetTensorImpl(), 4);
+                }
+        }
+    };
+    for (int level = 0; level < 4; ++level)
+        for (Py_ssize_t j = 0; j < (4 - level) * kAhead; ++j) stage(level, lo + j);
+    for (Py_ssize_t i = lo; i < hi; ++i) {
+        for (int level = 0; level < 4; ++level) stage(level, i + (4 - level) * kAhead);
+        PyObject* po = PyList_GET_ITEM(params, i);
+        if (!exact_tensor(po)) return false;
+        const at::Tensor& p = THPVariable_Unpack(po);
+        if (reinterpret_cast<uint64_t>(p.data_ptr()) != expect[3 * i]) return false;
+        const at::Tensor& g = p.grad();
+        const uint64_t want = expect[3 * i + 1];
+        if (!g.defined()) {
+            if (want != 0) return false;
+            continue;
+        }
+        if (want == 0 || g.layout() != at::kStrided || !g.is_contiguous() || g.numel() != p.numel() ||
+            reinterpret_cast<uint64_t>(g.data_ptr()) != want || (uint64_t)grad_code(g) != expect[3 * i + 2])
+            return false;
+    }
+    return true;
+}
+
+PyObject* verify_layout(PyObject*, PyObject* const* args, Py_ssize_t nargs) {
+    if (nargs != 3) {
+        PyErr_SetString(PyExc_TypeError, "verify_layout takes 3 arguments");
+        return nullptr;
+    }
+    PyObject* params = args[0];
+    if (!PyList_CheckExact(params)) {
+        PyErr_SetString(PyExc_TypeError, "params must be a list");
+        return nullptr;
+    }
+    const auto* expect = reinterpret_cast<const uint64_t*>(PyLong_AsUnsignedLongLong(args[1]));
+    const Py_ssize_t n = PyLong_AsSsize_t(args[2]);
+    if (PyErr_Occurred()) return nullptr;
+    if (PyList_GET_SIZE(params) != n || (n > 0 && !expect)) Py_RETURN_FALSE;
+    // The walk is bound by the latency of dependent loads, so long lists are split over a few
+    // threads.  The calling thread keeps the interpreter lock throughout: nothing can change the
+    // objects while the helpers read them, and the helpers call nothing of the interpreter.
+    const Py_ssize_t kPerThread = 2048;
+    const int threads = (int)std::min<Py_ssize_t>(8, std::max<Py_ssize_t>(1, n / kPerThread));
+    if (threads <= 1) {
+        if (verify_range(params, expect, 0, n)) Py_RETURN_TRUE;
+        Py_RETURN_FALSE;
+    }
+    std::vector<char> ok(threads, 0);
+    std::vector<std::thread> pool;
+    const Py_ssize_t per = (n + threads - 1) / threads;
+    for (int t = 1; t < threads; ++t)
+        pool.emplace_back([&, t] { ok[t] = verify_range(params, expect, t * per, std::min(n, (t + 1) * per)); });
+    ok[0] = verify_range(params, expect, 0, std::min(n, per));
+    for (auto& th : pool) th.join();
+    for (char c : ok)
+        if (!c) Py_RETURN_FALSE;
+    Py_RETURN_TRUE;
+}
+
 // set_types(torch.Tensor, torch.nn.Parameter): only objects of exactly these types take the fast path.
 PyObject* set_types(PyObject*, PyObject* args) {
     PyObject *a = nullptr, *b = nullptr;
@@ -274,6 +367,8 @@ PyObject* set_types(PyObject*, PyObject* args) {
 PyMethodDef methods[] = {
     {"gather_group", reinterpret_cast<PyCFunction>(reinterpret_cast<void (*)()>(gather_group)), METH_FASTCALL,
      "rt_tensor_desc rows of the plain tensors of one param group"},
+    {"verify_layout", reinterpret_cast<PyCFunction>(reinterpret_cast<void (*)()>(verify_layout)), METH_FASTCALL,
+     "whether every parameter and gradient of a recorded layout is still where it was"},
     {"set_types", set_types, METH_VARARGS, "register torch.Tensor and torch.nn.Parameter"},
     {nullptr, nullptr, 0, nullptr},
 };

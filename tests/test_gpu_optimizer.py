@@ -701,3 +701,58 @@ def test_state_placement_with_most_of_hbm_occupied_falls_back_quietly():
     finally:
         del hog
         torch.cuda.empty_cache()
+
+
+def test_frozen_layout_steps_like_the_full_path_and_notices_moved_gradients():
+    """assume_static_layout: after the first step the optimizer only checks that parameters and
+    gradients are where they were.  Same bits as an optimizer that gathers everything every step,
+    through a learning-rate change, a gradient that moves, one that vanishes, and state_dict()."""
+    rng = np.random.default_rng(11)
+    shapes = [(int(n),) for n in np.floor(np.exp(rng.uniform(0, np.log(3000), 396))).astype(int)] + [(64, 40)] * 4
+
+    def make(**kw):
+        ps, grads = _make_params(shapes, 7000)
+        for i, (p, g) in enumerate(zip(ps, grads)):
+            if i % 11 != 5:                  # some parameters never get a gradient
+                p.grad = g.clone()
+        return ps, ramtorch_amd.AdamW([{"params": ps[:300]}, {"params": ps[300:], "lr": 3e-4}], lr=1e-3,
+                                      storage_device="cuda", seed=9, **kw)
+
+    ps_a, a = make(assume_static_layout=True)
+    ps_b, b = make()
+
+    def same():
+        torch.cuda.synchronize()
+        for x, y in zip(ps_a, ps_b):
+            assert nmis(x.detach(), y.detach()) == 0
+            assert nmis(a.state[x]["ema"], b.state[y]["ema"]) == 0
+            assert nmis(a.state[x]["ema_squared"], b.state[y]["ema_squared"]) == 0
+
+    a.step(); b.step(); same()
+    assert a._frozen is not None and a._frozen["pending"] == 0
+    for k in range(3):
+        for opt in (a, b):
+            opt.param_groups[0]["lr"] *= 0.7          # a scheduler at work: re-read every step
+        for x, y in zip(ps_a, ps_b):                  # gradients accumulate in place
+            if x.grad is not None:
+                x.grad.mul_(1.25); y.grad.mul_(1.25)
+        a.step(); b.step(); same()
+        assert a._frozen is not None and a._frozen["pending"] == k + 1 and a.layout_refreezes == 0
+    sd_a, sd_b = a.state_dict(), b.state_dict()       # brings the lagging step counts up to date
+    assert [sd_a["state"][i]["step"] for i in sorted(sd_a["state"])] == [sd_b["state"][i]["step"] for i in sorted(sd_b["state"])]
+    # a gradient moves: caught, the step takes the full path and records the layout again
+    for ps in (ps_a, ps_b):
+        ps[7].grad = ps[7].grad.clone()
+    a.step(); b.step(); same()
+    assert a.layout_refreezes == 1 and a._frozen is not None
+    a.step(); b.step(); same()
+    assert a._frozen["pending"] == 1
+    # one vanishes, one appears
+    for ps in (ps_a, ps_b):
+        ps[8].grad = None
+        ps[5].grad = torch.full_like(ps[5], 1e-3)
+    a.step(); b.step(); same()
+    assert a.layout_refreezes == 2
+    a.unfreeze_layout()
+    assert [a.state[p]["step"] for p in ps_a] == [b.state[p]["step"] for p in ps_b]
+    a.step(); b.step(); same()

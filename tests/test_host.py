@@ -359,6 +359,61 @@ def test_copies_and_unpickled_optimizers_keep_their_configuration():
     assert opt.max_inflight_calls == 5 and opt.loss_scale == 4.0
 
 
+def test_layout_check_notices_every_kind_of_change():
+    """verify_layout (the per-step check of a recorded layout) on CPU tensors: true while nothing moved,
+    false for a moved / new / vanished / retyped / non-contiguous gradient and for a moved parameter."""
+    from ramtorch_amd import _gather as G
+    g = G.module()
+    if g is None or not hasattr(g, "verify_layout"):
+        pytest.skip("gather helper not built")
+    from ramtorch_amd import _native as N
+    ps = [torch.nn.Parameter(torch.zeros(6, 4, dtype=torch.bfloat16)) for _ in range(40)]
+    for i, p in enumerate(ps):
+        if i % 7:
+            p.grad = torch.ones(6, 4, dtype=torch.bfloat16)
+
+    def record():
+        e = np.zeros((len(ps), 3), np.uint64)
+        for i, p in enumerate(ps):
+            e[i, 0] = p.data_ptr()
+            if p.grad is not None:
+                e[i, 1] = p.grad.data_ptr()
+                e[i, 2] = {torch.bfloat16: N.RT_DT_BF16, torch.float32: N.RT_DT_F32, torch.float16: N.RT_DT_F16}[p.grad.dtype]
+        return e
+
+    def check(e):
+        return g.verify_layout(ps, e.ctypes.data, len(ps))
+
+    e = record()
+    assert check(e) is True
+    ps[3].grad.add_(1)                       # in-place accumulation keeps the layout
+    assert check(e) is True
+    keep = ps[3].grad
+    ps[3].grad = torch.ones(6, 4, dtype=torch.bfloat16)   # a new gradient tensor
+    assert check(e) is False
+    ps[3].grad = keep
+    assert check(e) is True
+    ps[0].grad = torch.ones(6, 4, dtype=torch.bfloat16)   # index 0 had none
+    assert check(e) is False
+    ps[0].grad = None
+    ps[5].grad = None                        # one vanished
+    assert check(e) is False
+    e = record()
+    assert check(e) is True
+    e2 = e.copy()
+    e2[8, 2] = N.RT_DT_F32                   # recorded with another dtype
+    assert check(e2) is False
+    base = torch.ones(4, 6, dtype=torch.bfloat16)
+    ps[9].grad = base.t()                    # same storage as a contiguous tensor would have, other strides
+    e3 = record()
+    assert check(e3) is False
+    ps[9].grad = torch.ones(6, 4, dtype=torch.bfloat16)
+    e = record()
+    ps[2].data = torch.zeros(6, 4, dtype=torch.bfloat16)  # the parameter moved
+    assert check(e) is False
+    assert g.verify_layout(ps[:-1], e.ctypes.data, len(ps)) is False   # list length differs
+
+
 def test_bench_refuses_more_than_one_gpu():
     """bench.py measures one GPU; asked for more it exits with a message instead of a number."""
     import subprocess
