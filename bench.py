@@ -171,8 +171,24 @@ def cpu_baseline():
 
 
 # ---- GPU workloads ----------------------------------------------------------------------------
-def build_resident(shapes, *, g_dtype, device, seed=1234):
+def build_resident(shapes, *, g_dtype, device, seed=1234, flat=False):
     import torch
+    gdt = torch.float32 if g_dtype == torch.float32 else torch.bfloat16
+    if flat:
+        # thousands of short tensors: carved out of one parameter buffer and one gradient buffer at
+        # 512-byte steps, which is how torch's allocator packs small tensors anyway, and filled by two
+        # kernels instead of tens of thousands
+        offs, total = [], 0
+        for shp in shapes:
+            offs.append(total)
+            total += (numel(shp) + 255) // 256 * 256
+        pbuf = fill_tensor((total,), "p", seed, torch.bfloat16, device)
+        gbuf = fill_tensor((total,), "g", seed + 1, gdt, device)
+        if g_dtype == torch.float32:
+            gbuf.mul_(1024.0)
+        params = [torch.nn.Parameter(pbuf[o:o + numel(shp)].view(shp), requires_grad=False) for o, shp in zip(offs, shapes)]
+        grads = [gbuf[o:o + numel(shp)].view(shp) for o, shp in zip(offs, shapes)]
+        return params, grads
     # parameters first, gradients afterwards: the order a framework allocates them in (model
     # construction, then the backward pass), so a parameter and its gradient are not neighbours
     params, grads = [], []
@@ -180,8 +196,7 @@ def build_resident(shapes, *, g_dtype, device, seed=1234):
         params.append(torch.nn.Parameter(fill_tensor(shp, "p", seed + 4 * i, torch.bfloat16, device),
                                          requires_grad=False))
     for i, shp in enumerate(shapes):
-        g = fill_tensor(shp, "g", seed + 4 * i + 1, torch.float32 if g_dtype == torch.float32 else torch.bfloat16,
-                        device)
+        g = fill_tensor(shp, "g", seed + 4 * i + 1, gdt, device)
         if g_dtype == torch.float32:
             g.mul_(1024.0)
         grads.append(g)
@@ -190,9 +205,19 @@ def build_resident(shapes, *, g_dtype, device, seed=1234):
 
 def set_states(opt, params, first_step, warmup, dev):
     import torch
+    pools = getattr(opt, "_state_pools", None) or {}
+    pooled = "ema" in pools and all(s is not None for s in pools.get("slots", [None]))
+    if pooled and len(params) > 1000:
+        # all states are views into two pools: fill the pools, not 2 x 20 000 views (padding included; harmless)
+        for k, key in ((2, "ema"), (3, "ema_squared")):
+            dt = opt.state[params[0]][key].dtype
+            view = pools[key].view(dt)
+            view.copy_(fill_tensor((view.numel(),), "m" if key == "ema" else "v", 1234 + k, dt, dev))
     for i, p in enumerate(params):
         st = opt.state[p]
         st["step"] = first_step - 1 - warmup
+        if pooled and len(params) > 1000:
+            continue
         # the states stay the tensors the optimizer allocated (and placed); only their contents are set
         st["ema"].copy_(fill_tensor(p.shape, "m", 1234 + 4 * i + 2, torch.bfloat16, dev))
         st["ema_squared"].copy_(fill_tensor(p.shape, "v", 1234 + 4 * i + 3, st["ema_squared"].dtype, dev))
@@ -242,11 +267,12 @@ def run_resident(wl, args, steps, warmup, *, full):
         first_step = 10
     elif wl == "small":
         shapes = small_tensor_shapes()
+        opt_kw.update(state_pool_min_bytes=0)   # states as views into two pools, like the large sets
     else:  # mixed
         shapes = llama3_8b_shapes(args.layers)
         g_dtype = torch.float32
         opt_kw.update(loss_scale=1024.0, max_grad_norm=1.0, ema_squared_dtype=torch.float32)
-    params, grads = build_resident(shapes, g_dtype=g_dtype, device=dev)
+    params, grads = build_resident(shapes, g_dtype=g_dtype, device=dev, flat=wl == "small")
     total = sum(numel(s) for s in shapes)
     opt = ramtorch_amd.AdamW(params, dtype=torch.bfloat16, **HP, **opt_kw)
     set_states(opt, params, first_step, warmup, dev)
@@ -291,7 +317,7 @@ def run_resident(wl, args, steps, warmup, *, full):
     if full:
         # The same state tensors allocated one by one, as the reference allocates them, instead of
         # in two pools placed in different HBM regions: what the placement is worth on this box.
-        if args.state_placement == "auto" and opt.state_placement_report is not None:
+        if args.state_placement == "auto" and opt.state_placement_report is not None and len(params) < 1000:
             plain = ramtorch_amd.AdamW(params, dtype=torch.bfloat16, **HP, **dict(opt_kw, state_placement="plain"))
             for p in params:
                 plain.state[p]["step"] = first_step - 1

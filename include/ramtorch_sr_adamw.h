@@ -267,6 +267,7 @@ int rt_host_link_probe(rt_handle* h, uint64_t bytes, int reps, double out[3]);
  * without going through -- and leaving blocks behind in -- the caller's own
  * caching allocator.  Nothing in the reference corresponds to it.
  * rt_dev_hold returns RT_ENOMEM when the device has no such block left.
+ * rt_dev_release accepts h == NULL (the block's device is found by its address).
  */
 int rt_dev_hold(rt_handle* h, uint64_t bytes, void** out);
 int rt_dev_release(rt_handle* h, void* p);

@@ -39,7 +39,7 @@ def noise_to_i32(noise_i16: torch.Tensor) -> torch.Tensor:
 
 @torch.no_grad()
 def reference_step_ops(p, grad, ema, ema_squared, *, lr, betas, eps, weight_decay, step, noise=None,
-                       compute_device=None):
+                       compute_device=None, centralization=0):
     """In-place step on ``p`` / ``ema`` / ``ema_squared``; ``step`` is the value
     after the increment (adamw.py:177).  ``noise`` = three int16 tensors, or
     None to draw as the reference does (seeds step+42 / +69 / +420).
@@ -57,6 +57,9 @@ def reference_step_ops(p, grad, ema, ema_squared, *, lr, betas, eps, weight_deca
         ema_fp32 = ema_fp32.clone()
     if ema_squared_fp32 is ema_squared:
         ema_squared_fp32 = ema_squared_fp32.clone()
+
+    if centralization != 0:
+        g.sub_(g.mean(dim=tuple(range(1, g.dim())), keepdim=True).mul_(centralization))   # :179-184
 
     beta1, beta2 = betas
     bias_correction = 1 - beta1 ** step                                               # :186

@@ -332,5 +332,10 @@ def streamed_plan(descs, n: int, chunk_elems: int):
     return [tuple(buf[5 * i:5 * i + 5]) for i in range(k.value)]
 
 
+def dev_release(addr: int) -> None:
+    """Give a block of rt_dev_hold back without a handle (hipFree finds the device by the address)."""
+    check(lib().rt_dev_release(None, ctypes.c_void_p(addr)))
+
+
 def sr_copy(target_ptr, source_ptr, numel, noise_ptr, seed, stream=0) -> None:
     check(lib().rt_sr_copy(target_ptr, source_ptr, numel, noise_ptr, seed, stream))

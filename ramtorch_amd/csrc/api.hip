@@ -1493,10 +1493,9 @@ int rt_dev_hold(rt_handle* h, uint64_t bytes, void** out) {
 }
 
 int rt_dev_release(rt_handle* h, void* p) {
-    if (!h) return fail(RT_EINVAL, "handle is NULL");
     if (!p) return RT_OK;
-    HIP_TRY(hipSetDevice(h->device));
-    HIP_TRY(hipFree(p));
+    if (h) HIP_TRY(hipSetDevice(h->device));
+    HIP_TRY(hipFree(p));  // the runtime finds the owning device by the address
     return RT_OK;
 }
 

@@ -51,6 +51,26 @@ def split_probe(handle: N.Handle, a_ptr: int, a_bytes: int, b_ptr: int, b_bytes:
     return out
 
 
+class _HeldBlock:
+    """A device block held through the library, seen by torch as a 1-D uint8 tensor (``tensor()``).
+    The tensor and every view of it keep this object alive; the block is given back when the last
+    of them has gone."""
+
+    def __init__(self, addr: int, nbytes: int, device: torch.device):
+        self.addr, self.nbytes, self.device = addr, nbytes, device
+        self.__cuda_array_interface__ = {"shape": (nbytes,), "typestr": "|u1", "data": (addr, False), "version": 2,
+                                         "strides": None}
+
+    def tensor(self) -> torch.Tensor:
+        return torch.as_tensor(self, device=self.device)
+
+    def __del__(self):
+        try:
+            N.dev_release(self.addr)
+        except Exception:
+            pass  # interpreter shutdown: the process is about to return the memory anyway
+
+
 def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: int, *,
                min_gain: float = 1.05, filler_bytes: int = 2 * GIB, step_bytes: int = 16 * GIB,
                max_filler_bytes: int = 112 * GIB, max_fraction_of_free: float = 0.5, max_seconds: float = 8.0,
@@ -62,14 +82,17 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
     The place right behind the first pool is tried first.  Unless the probe shows the gain there
     (mean over the beginning, middle and end of the pools), memory is occupied with filler blocks
     (memory the driver hands out in moderate blocks follows in physical address order; one huge
-    block does not) and after every ``step_bytes`` of them the next place is tried, until one shows
+    block does not) and after every ``step_bytes`` of them the place a block of the pool's size
+    gets is tried, until one shows
     the gain or the search runs out of ``max_filler_bytes`` (a region is 96 GiB),
     ``max_fraction_of_free`` of the memory that was free at the start, or ``max_seconds``.
 
     Everything the search occupies on the way -- fillers and the places it tried -- is held through
-    the library (``rt_dev_hold``), not through torch, and given back before this returns: torch's
-    caching allocator is left as it was, apart from the two pools.  With little free memory the
-    search simply ends early and the second pool lands wherever torch puts it (``placed: False``)."""
+    the library (``rt_dev_hold``), not through torch, and given back before this returns; the place
+    that shows the gain stays held and *is* the second pool (a torch tensor over that block, which
+    goes back to the driver when its last view has gone).  torch's caching allocator only ever sees
+    the first pool.  With little free memory the search simply ends early and the second pool is an
+    ordinary torch allocation, wherever that lands (``placed: False``)."""
     stream = torch.cuda.current_stream(device).cuda_stream
 
     def zeros(nbytes):
@@ -108,23 +131,21 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
             if log:
                 log(f"{held_bytes / GIB:.0f} GiB occupied: same {same:.0f} GB/s, split {cross:.0f} GB/s")
             if full:
-                # give the place back and let torch take it; then make sure that it did
-                handle.dev_release(cand)
-                b = zeros(bytes_b)
-                same, cross, full = summary(split_probe(handle, a.data_ptr(), bytes_a, b.data_ptr(), bytes_b, device,
-                                                        stream))
-                report.update(placed=full, filler_GiB=held_bytes / GIB, same_GBps=same, cross_GBps=cross)
+                # this very block becomes the second pool: nothing is released and allocated again
+                b = _HeldBlock(cand, bytes_b, device).tensor()
+                b.zero_()
+                report.update(placed=True, filler_GiB=held_bytes / GIB, same_GBps=same, cross_GBps=cross)
                 break
-            # not here: the block stays where it is as a filler, and more follow
-            held.append(cand)
-            held_bytes += bytes_b
-            want = max(0, step_bytes - bytes_b)
+            # Not here.  The place is given back and occupied again, together with what follows it,
+            # by moderate filler blocks: those the driver hands out in physical address order, which
+            # it does not do for one huge block.
+            handle.dev_release(cand)
             free, _ = torch.cuda.mem_get_info(device)
-            if (held_bytes + want + bytes_b > budget or want + 2 * bytes_b + 4 * GIB > free
+            if (held_bytes + step_bytes > budget or step_bytes + bytes_b + 4 * GIB > free
                     or time.monotonic() - t0 > max_seconds):
                 break
             try:
-                for _ in range(want // filler_bytes):
+                for _ in range(max(1, step_bytes // filler_bytes)):
                     held.append(handle.dev_hold(filler_bytes))
                     held_bytes += filler_bytes
             except N.NativeError:

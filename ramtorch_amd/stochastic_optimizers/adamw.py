@@ -108,7 +108,10 @@ class AdamW(Optimizer):
             "reference" draws it the way the reference does -- three ``torch.randint``
             tensors per parameter from generators seeded ``step + 42 / 69 / 420``
             (adamw.py:10-21, 206-218) -- and feeds it to the kernel as explicit noise, so
-            that a run is bit-identical to ``ramtorch.AdamW`` under the same torch build.
+            that a run is bit-identical to ``ramtorch.AdamW`` under the same torch build
+            (with ``centralization`` the row means are then taken with torch's own ``mean``,
+            as the reference takes them; the default path uses the library's row-mean kernel,
+            whose sums agree with torch's to about 2e-6 relative, not bit for bit).
             A verification mode: it costs the three draws and their memory.
         state_placement: "auto" (default) or "plain".  With GPU-resident states of at least
             ``state_pool_min_bytes`` per kind, "auto" carves all ``ema`` tensors out of one
@@ -556,8 +559,14 @@ class AdamW(Optimizer):
                     rows = g.shape[0] if g.dim() >= 2 else 1
                     row_len = g.numel() // rows if rows else 0
                     if g.numel():
-                        with torch.cuda.device(dev):
-                            e.row_mean = F.row_means(_handle(dev), g, rows, row_len, inv_loss_scale)
+                        if getattr(self, "noise_source", "philox") == "reference" and inv_loss_scale == 1.0:
+                            # the verification mode reproduces the reference bit for bit: the means come
+                            # from the very call the reference makes (a sum's bits depend on its order)
+                            g32 = g.to(torch.float32)
+                            e.row_mean = g32.mean(dim=tuple(range(1, g32.dim())), keepdim=True).reshape(-1).contiguous()
+                        else:
+                            with torch.cuda.device(dev):
+                                e.row_mean = F.row_means(_handle(dev), g, rows, row_len, inv_loss_scale)
                         e.row_len = row_len
                 if noise is not None and p in noise:
                     e.noise = tuple(noise[p])

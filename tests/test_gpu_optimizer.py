@@ -756,3 +756,21 @@ def test_frozen_layout_steps_like_the_full_path_and_notices_moved_gradients():
     a.unfreeze_layout()
     assert [a.state[p]["step"] for p in ps_a] == [b.state[p]["step"] for p in ps_b]
     a.step(); b.step(); same()
+
+
+@pytest.mark.parametrize("shape", [(37, 24), (4, 3, 10), (129,)])
+def test_reference_noise_mode_with_centralization_is_bit_identical_to_the_reference_step(shape):
+    """noise_source="reference" takes the row means with torch's own mean, as adamw.py:179-184 does, so the
+    whole step equals the reference's op sequence bit for bit (its own randint noise included)."""
+    ps, grads = _make_params([shape], 8100)
+    p = ps[0]
+    ref_p = p.detach().clone()
+    ref_m, ref_v = torch.zeros_like(ref_p), torch.zeros_like(ref_p)
+    opt = ramtorch_amd.AdamW([p], storage_device="cuda", centralization=0.5, noise_source="reference", **HP0)
+    for step in (1, 2):
+        p.grad = (grads[0].float() * (1.0 + 0.3 * step)).bfloat16()
+        opt.step()
+        torch.cuda.synchronize()
+        torch_ops.reference_step_ops(ref_p, p.grad, ref_m, ref_v, step=step, noise=None, centralization=0.5, **HP0)
+        assert nmis(p.detach(), ref_p) == 0, f"step {step}"
+        assert nmis(opt.state[p]["ema"], ref_m) == 0 and nmis(opt.state[p]["ema_squared"], ref_v) == 0
