@@ -57,8 +57,12 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the dominant update kernel.  NOT measured in this run: rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE figures of earlier runs of this script (each scaled by what the same
 # counter reads for a plain kernel of known size in the same run), kept under profiles/.
+_TRAFFIC_FILE = "profiles/sr_adamw_kernels_hbm_traffic.txt"
 OFFLINE_TRAFFIC = {
-    "llama8b": (112_546_390_426, "profiles/sr_adamw_fast_kernel_llama8b_hbm_traffic.txt"),
+    "llama8b": (112_422_266_998, _TRAFFIC_FILE),
+    "mixed": (160_597_606_615, _TRAFFIC_FILE),      # the update launch; its norm pass fetches 32 120 545 889 B more
+    "small": (1_090_935_301, _TRAFFIC_FILE),
+    "cfg0": (335_774_529, _TRAFFIC_FILE),
 }
 HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
 METRIC = "SR-AdamW step: params/sec + achieved HBM GB/s (% of peak), 8B bf16 set, 1 GPU"

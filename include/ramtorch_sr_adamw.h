@@ -221,8 +221,9 @@ int rt_sr_copy(void* target_bf16, const float* source, uint64_t numel, const voi
 
 /*
  * Timing of rt_step_multi launches on this handle, measured with HIP events
- * recorded on the launch stream around the update kernels only (a pair per
- * launch, nothing is read or waited for while launches are being queued).
+ * attached to the update kernels' own dispatches on the launch stream (start
+ * of the first kernel of a call, end of its last; a pair per call, nothing is
+ * read or waited for while launches are being queued).
  * Measurement only; nothing in the reference corresponds to it.
  *   rt_set_timing(h, 1): start recording (and forget earlier launches); (h, 0): stop
  *   rt_last_kernel_ms:   duration of the most recent timed launch; blocks until it has finished

@@ -2,6 +2,7 @@
 // checks, the device-side tensor / chunk tables, kernel dispatch by dtype
 // combination, and the streamed (host-resident) pipeline.  gfx950 only.
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <algorithm>
 #include <chrono>
@@ -527,8 +528,12 @@ static int stage_image(rt_handle* h, const Plan& plan, const uint8_t* img, uint6
 }
 
 // Enqueues the update kernels of one table image that already sits in device memory at `base`.
+// `t_begin` / `t_end` (timed launches): events attached to the dispatches themselves -- the first
+// kernel's start and the last kernel's end -- so that what is read back is kernel time, without the
+// few microseconds a marker before and after a dispatch adds.
 static int enqueue_kernels(const Plan& plan, const uint8_t* base, uint64_t seed, int noise_mode,
-                           const float* d_clip_coef, const uint32_t* d_skip, hipStream_t stream) {
+                           const float* d_clip_coef, const uint32_t* d_skip, hipStream_t stream,
+                           hipEvent_t t_begin = nullptr, hipEvent_t t_end = nullptr) {
     LaunchArgs a;
     memset(&a, 0, sizeof(a));
     a.tensors = (const DevTensor*)(base + plan.off_tensors);
@@ -539,6 +544,12 @@ static int enqueue_kernels(const Plan& plan, const uint8_t* base, uint64_t seed,
     a.seed_hi = (uint32_t)(seed >> 32);
     a.use_ks = plan.n_sets == 1 ? 1u : 0u;
     a.ks = plan.first_set;
+    struct Launch {
+        MultiKernel kernel;
+        uint32_t grid;
+        LaunchArgs args;
+    };
+    std::vector<Launch> launches;
     for (const Batch& b : plan.batches) {
         KernelPair k;
         if (b.combo == kComboAny) {
@@ -560,14 +571,18 @@ static int enqueue_kernels(const Plan& plan, const uint8_t* base, uint64_t seed,
         if (a.n_piece_wgs != 0 && b.n_units != 0)
             a.piece_rate = (uint32_t)((((uint64_t)a.n_piece_wgs << 32) + grid - 1) / grid);  // < 2^32: n_piece_wgs < grid
         if (grid > kMaxGrid || b.n_generic > kMaxGrid) return fail(RT_EUNSUPPORTED, "too many workgroups in one launch");
-        if (grid) {
-            hipLaunchKernelGGL(k.fast, dim3((uint32_t)grid), dim3(kThreads), 0, stream, a);
-            HIP_TRY(hipGetLastError());
-        }
-        if (b.n_generic) {
-            hipLaunchKernelGGL(k.generic, dim3(b.n_generic), dim3(kThreads), 0, stream, a);
-            HIP_TRY(hipGetLastError());
-        }
+        if (grid) launches.push_back(Launch{k.fast, (uint32_t)grid, a});
+        if (b.n_generic) launches.push_back(Launch{k.generic, b.n_generic, a});
+    }
+    for (size_t i = 0; i < launches.size(); ++i) {
+        const Launch& l = launches[i];
+        const hipEvent_t e0 = i == 0 ? t_begin : nullptr;
+        const hipEvent_t e1 = i + 1 == launches.size() ? t_end : nullptr;
+        if (e0 || e1)
+            hipExtLaunchKernelGGL(l.kernel, dim3(l.grid), dim3(kThreads), 0, stream, e0, e1, 0, l.args);
+        else
+            hipLaunchKernelGGL(l.kernel, dim3(l.grid), dim3(kThreads), 0, stream, l.args);
+        HIP_TRY(hipGetLastError());
     }
     return RT_OK;
 }
@@ -630,17 +645,11 @@ static int launch_update(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, 
     TableSlot* slot = nullptr;
     int rc = stage_image(h, plan, lc.image.data(), lc.gen, stream, &slot);
     if (rc != RT_OK) return rc;
-    std::pair<hipEvent_t, hipEvent_t>* tp = nullptr;
-    if (h->timing) {
-        tp = &h->tring[h->timed_launches % kTimingRing];
-        HIP_TRY(hipEventRecord(tp->first, stream));
-    }
-    rc = enqueue_kernels(plan, (const uint8_t*)slot->dev.ptr, seed, noise_mode, d_clip_coef, d_skip, stream);
+    std::pair<hipEvent_t, hipEvent_t>* tp = h->timing ? &h->tring[h->timed_launches % kTimingRing] : nullptr;
+    rc = enqueue_kernels(plan, (const uint8_t*)slot->dev.ptr, seed, noise_mode, d_clip_coef, d_skip, stream,
+                         tp ? tp->first : nullptr, tp ? tp->second : nullptr);
     if (rc != RT_OK) return rc;
-    if (tp) {
-        HIP_TRY(hipEventRecord(tp->second, stream));
-        ++h->timed_launches;
-    }
+    if (tp) ++h->timed_launches;
     HIP_TRY(hipEventRecord(slot->done, stream));
     slot->in_flight = true;
     return RT_OK;

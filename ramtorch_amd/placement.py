@@ -80,7 +80,7 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
     (pool_a, pool_b, report).
 
     The place right behind the first pool is tried first.  Unless the probe shows the gain there
-    (mean over the beginning, middle and end of the pools), memory is occupied with filler blocks
+    (at the beginning, in the middle and at the end of the pools alike), memory is occupied with filler blocks
     (memory the driver hands out in moderate blocks follows in physical address order; one huge
     block does not) and after every ``step_bytes`` of them the place a block of the pool's size
     gets is tried, until one shows
@@ -103,13 +103,23 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
     free0, _ = torch.cuda.mem_get_info(device)
     a = zeros(bytes_a)
     budget = min(max_filler_bytes, int(max_fraction_of_free * max(0, free0 - bytes_a - bytes_b)))
-    held, held_bytes = [], 0      # addresses of blocks held through the library
+    held, held_bytes = [], 0      # addresses of filler blocks held through the library
+    best = None                   # (address, same, cross) of the best place seen that fell short of min_gain
     b = None
 
     def summary(r):
+        # mean rates, and whether the gain shows at every probed position (a block that straddles
+        # two regions shows it at some of them only)
         same = sum(x[0] for x in r) / len(r)
         cross = sum(x[1] for x in r) / len(r)
-        return same, cross, cross >= min_gain * same
+        return same, cross, all(x[1] >= min_gain * x[0] for x in r)
+
+    def adopt(addr, same, cross, placed):
+        # this very block becomes the second pool: nothing is released and allocated again
+        t = _HeldBlock(addr, bytes_b, device).tensor()
+        t.zero_()
+        report.update(placed=placed, filler_GiB=held_bytes / GIB, same_GBps=same, cross_GBps=cross)
+        return t
 
     try:
         while b is None:
@@ -126,20 +136,24 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
                 break
             same, cross, full = summary(res)
             report["tries"] += 1
-            if report["cross_GBps"] is None or cross > report["cross_GBps"]:
+            if report["cross_GBps"] is None:
                 report.update(same_GBps=same, cross_GBps=cross)
             if log:
                 log(f"{held_bytes / GIB:.0f} GiB occupied: same {same:.0f} GB/s, split {cross:.0f} GB/s")
             if full:
-                # this very block becomes the second pool: nothing is released and allocated again
-                b = _HeldBlock(cand, bytes_b, device).tensor()
-                b.zero_()
-                report.update(placed=True, filler_GiB=held_bytes / GIB, same_GBps=same, cross_GBps=cross)
+                b = adopt(cand, same, cross, True)
                 break
-            # Not here.  The place is given back and occupied again, together with what follows it,
-            # by moderate filler blocks: those the driver hands out in physical address order, which
-            # it does not do for one huge block.
-            handle.dev_release(cand)
+            # Not here, or only in part (a block that straddles two regions shows the gain at some of
+            # the probed positions).  The best such place stays held in case nothing better turns up;
+            # any other is given back and occupied again, together with what follows it, by moderate
+            # filler blocks: those the driver hands out in physical address order, which it does not
+            # do for one huge block.
+            if best is None or cross / same > best[2] / best[1]:
+                if best is not None:
+                    handle.dev_release(best[0])
+                best = (cand, same, cross)
+            else:
+                handle.dev_release(cand)
             free, _ = torch.cuda.mem_get_info(device)
             if (held_bytes + step_bytes > budget or step_bytes + bytes_b + 4 * GIB > free
                     or time.monotonic() - t0 > max_seconds):
@@ -150,9 +164,14 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
                     held_bytes += filler_bytes
             except N.NativeError:
                 break
+        if b is None and best is not None and best[2] >= 1.01 * best[1]:
+            b = adopt(best[0], best[1], best[2], False)   # part of the gain is better than none
+            best = None
     finally:
         for addr in held:
             handle.dev_release(addr)
+        if best is not None:
+            handle.dev_release(best[0])
     if b is None:
         b = zeros(bytes_b)
     report["seconds"] = time.monotonic() - t0
