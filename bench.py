@@ -28,6 +28,9 @@ ema~N(0,1e-4), ema_squared=N(0,1e-3)^2, stored bf16):
   small     20 000 small tensors (length log-uniform in [1,4096]) + 64 x 1024x1024
   mixed     Llama-3-8B shapes; bf16 p and ema, fp32 ema_squared, fp32 grads scaled
             by 1024 and unscaled in-kernel, global-norm clip to 1.0
+  central   the default set with centralization=1.0 (adamw.py:179-184): one row-mean
+            pass per matrix (2 B per element read) and the update through the
+            kernel that subtracts the means (14 B per element + 4 B per row)
   streamed  Llama-3-8B shapes with p/ema/ema_squared in pinned host memory,
             bf16 grads on the GPU, 256 MB chunks (--stream-gb bounds the host set)
   hooked    the same set, but each tensor is updated by AdamW.step_param() as a
@@ -66,10 +69,10 @@ OFFLINE_TRAFFIC = {
 }
 HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
 METRIC = "SR-AdamW step: params/sec + achieved HBM GB/s (% of peak), 8B bf16 set, 1 GPU"
-RESIDENT = ("llama8b", "cfg0", "small", "mixed")
+RESIDENT = ("llama8b", "cfg0", "small", "mixed", "central")
 HOST = ("streamed", "hooked", "offload_ref")
-UPDATE_BYTES = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 20}   # per element, update launch only
-STEP_BYTES = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 24, "streamed": 12, "hooked": 12, "offload_ref": 14}
+UPDATE_BYTES = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 20, "central": 14}   # per element, update launch only
+STEP_BYTES = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 24, "central": 16, "streamed": 12, "hooked": 12, "offload_ref": 14}
 
 
 # ---- workload shapes -------------------------------------------------------------------------
@@ -266,6 +269,9 @@ def run_resident(wl, args, steps, warmup, *, full):
     g_dtype = torch.bfloat16
     if wl == "llama8b":
         shapes = llama3_8b_shapes(args.layers)
+    elif wl == "central":
+        shapes = llama3_8b_shapes(args.layers)
+        opt_kw.update(centralization=1.0)
     elif wl == "cfg0":
         shapes = [(4096, 4096)]
         first_step = 10
@@ -304,7 +310,7 @@ def run_resident(wl, args, steps, warmup, *, full):
                 "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic[0] if traffic else None,
                 "traffic_source": (f"not measured in this run: rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of an earlier "
                                    f"run, {traffic[1]}") if traffic else None,
-                "kernel": "sr_adamw_fast_wide_kernel" if wl == "mixed" else "sr_adamw_fast_kernel",
+                "kernel": {"mixed": "sr_adamw_fast_wide_kernel", "central": "sr_adamw_generic_kernel"}.get(wl, "sr_adamw_fast_kernel"),
                 "kernel_ms": k_ms, "kernel_launches_timed": len(ks), "algorithmic_bytes_per_launch": upd_bytes}
     out = {"ms_per_step": ms_per_step, "elements_per_s": total / (ms_per_step * 1e-3),
            "achieved_GBps_wall": STEP_BYTES[wl] * total / (ms_per_step * 1e-3) / 1e9,
@@ -415,11 +421,16 @@ def run_host(workloads, args, steps, warmup):
             one_step = lambda: opt.step(grads=cpu_grads)
         else:
             one_step = lambda: opt.step(grads=gmap)
+        bounce0 = handle.streamed_bounce_stats()
         ms_per_step, _ = timed_steps(one_step, steps, warmup, handle, False)
+        bounce1 = handle.streamed_bounce_stats()
         up = {"streamed": 6.0, "hooked": 6.0, "offload_ref": 8.0}[wl] * total
         down = 6.0 * total
         secs = ms_per_step * 1e-3
         info = {"h2d_GBps": up / secs / 1e9, "d2h_GBps": down / secs / 1e9, "host_bytes_up": up, "host_bytes_down": down}
+        if bounce1["calls"] != bounce0["calls"]:
+            # host arrays that are not pinned went up through the library's pinned bounce buffers
+            info["bounced_bytes_per_step"] = (bounce1["bytes"] - bounce0["bytes"]) / (steps + warmup)
         if link is None:
             # same-run pinned-copy peaks with the same chunk size, each direction alone and both at
             # once (what the pipeline does in steady state), on the library's own copy streams

@@ -139,6 +139,15 @@ int rt_step_multi(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const r
  * Results are bit-identical to rt_step_multi on the same data.
  * d_clip_coef / d_skip: as for rt_step_multi (device pointers, may be NULL);
  * they must be final for work queued on `stream` before the call.
+ * Host arrays need not be pinned: the gradients that ramtorch's Linear.backward
+ * leaves in ordinary CPU memory (linear.py:416-427, shipped up at adamw.py:167)
+ * are copied into pinned bounce buffers of the handle (4 per array, one chunk
+ * each) by a few host threads while earlier chunks are on the link, and the
+ * call then hands the pipeline one chunk at a time.  RT_STREAM_BOUNCE_THREADS
+ * in the environment sets the number of threads (default 4; 0 leaves such
+ * copies to the runtime, which stages them while the calling thread waits).
+ * Updated arrays that go back into memory that is not pinned are always left
+ * to the runtime.
  */
 int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
                      uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems,
@@ -288,6 +297,13 @@ int rt_selftest_sqrt(rt_handle* h, uint64_t* mismatches);
  * out[0] = bytes H2D, out[1] = bytes D2H, out[2] = wall seconds of the call.
  */
 int rt_streamed_stats(rt_handle* h, double out[3]);
+
+/*
+ * How often the streamed path met host arrays that are not pinned, since the
+ * handle was created: out[0] = calls that went through the bounce buffers,
+ * out[1] = bytes the host threads copied into them.
+ */
+int rt_streamed_bounce_stats(rt_handle* h, uint64_t out[2]);
 
 /*
  * Per-chunk timeline of the most recent rt_step_streamed made while timing was

@@ -30,6 +30,7 @@ EXPORTS = (
     "rt_stream_probe", "rt_streamed_timeline", "rt_streamed_plan",
     "rt_step_streamed_async", "rt_streamed_wait", "rt_streamed_completed",
     "rt_grad_norm_static", "rt_host_link_probe", "rt_selftest_sqrt", "rt_dev_hold", "rt_dev_release",
+    "rt_streamed_bounce_stats",
 )
 
 
@@ -153,6 +154,8 @@ def lib() -> ctypes.CDLL:
     L.rt_streamed_plan.argtypes = [descs, u32, u64, ctypes.POINTER(u64), u32, ctypes.POINTER(u32)]
     L.rt_streamed_stats.restype = i32
     L.rt_streamed_stats.argtypes = [vp, ctypes.POINTER(ctypes.c_double)]
+    L.rt_streamed_bounce_stats.restype = i32
+    L.rt_streamed_bounce_stats.argtypes = [vp, ctypes.POINTER(ctypes.c_uint64)]
     v = L.rt_version()
     if v != ABI_VERSION:
         raise RuntimeError(f"{LIB_PATH} has ABI version {v}, this package expects {ABI_VERSION}; rebuild it")
@@ -308,6 +311,13 @@ class Handle:
         with self._lock:
             check(lib().rt_streamed_stats(self.ptr, out))
         return {"bytes_h2d": out[0], "bytes_d2h": out[1], "seconds": out[2]}
+
+    def streamed_bounce_stats(self):
+        """Calls that met host arrays that are not pinned, and the bytes host threads copied for them."""
+        out = (ctypes.c_uint64 * 2)()
+        with self._lock:
+            check(lib().rt_streamed_bounce_stats(self.ptr, out))
+        return {"calls": int(out[0]), "bytes": int(out[1])}
 
 
 _live_handles: "weakref.WeakSet[Handle]" = weakref.WeakSet()

@@ -19,7 +19,7 @@ LIB_DIR = os.path.join(HERE, "_lib")
 LIB_PATH = os.path.join(LIB_DIR, "libramtorch_sr_adamw.so")
 
 SOURCES = ["api.hip"]
-HEADERS = ["kernels.h", "device_types.h", os.path.join("..", "..", "include", "ramtorch_sr_adamw.h")]
+HEADERS = ["kernels.h", "device_types.h", "copy_pool.h", os.path.join("..", "..", "include", "ramtorch_sr_adamw.h")]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

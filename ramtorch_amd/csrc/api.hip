@@ -14,11 +14,13 @@
 #include <cstdint>
 #include <cstring>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <new>
 #include <thread>
 #include <vector>
 
+#include "copy_pool.h"
 #include "kernels.h"
 
 using namespace rt;
@@ -55,6 +57,9 @@ constexpr size_t kTablePoolBytes = 64 << 10;
 constexpr int kNormPartials = 2048;  // workgroups of the norm pass
 constexpr size_t kTimingRing = 256;   // timed launches whose durations can be read back
 constexpr uint64_t kMaxGrid = 0x7FFFFFFFull;  // workgroups of one launch (one per chunk of 8192 elements)
+constexpr int kStageBufs = 2;        // device staging buffers per array (chunks in different stages of the pipeline)
+constexpr int kBounce = 4;           // pinned bounce buffers per array for host arrays that are not pinned
+constexpr uint64_t kPacedInFlight = 2;  // chunks on the streams while the host feeds the pipeline chunk by chunk
 
 struct DevBuf {
     void* ptr = nullptr;
@@ -76,10 +81,10 @@ struct TableSlot {
 struct Streamed {
     hipStream_t h2d = nullptr, comp = nullptr, d2h = nullptr;
     hipEvent_t start = nullptr;
-    hipEvent_t h2d_done[2] = {nullptr, nullptr};
-    hipEvent_t comp_done[2] = {nullptr, nullptr};
-    hipEvent_t d2h_done[2] = {nullptr, nullptr};
-    DevBuf stage[4][2];  // [p,g,m,v][buffer]
+    hipEvent_t h2d_done[kStageBufs] = {};
+    hipEvent_t comp_done[kStageBufs] = {};
+    hipEvent_t d2h_done[kStageBufs] = {};
+    DevBuf stage[4][kStageBufs];  // [p,g,m,v][buffer]
     // Table images of every chunk of one call, back to back.  A pool, because an
     // asynchronous call may still be running when the next one builds its tables; an
     // entry is free again once the ticket of the call that used it has been published,
@@ -94,8 +99,8 @@ struct Streamed {
     };
     std::vector<TableRing> ring;
     // The pipeline state survives across calls so that asynchronous calls chain correctly:
-    uint64_t seq = 0;                      // chunks enqueued so far; chunk `seq` uses buffer seq & 1
-    bool used_buf[2] = {false, false};     // buffer has a D2H whose completion the next H2D must await
+    uint64_t seq = 0;                      // chunks enqueued so far; chunk `seq` uses buffer seq % kStageBufs
+    bool used_buf[kStageBufs] = {};        // buffer has a D2H whose completion the next H2D must await
     bool pending = false;                  // work enqueued since the last wait
     // Tickets: a one-thread kernel behind the last D2H copy of a call writes the call's number
     // into a word of pinned host memory; the host learns about completion by reading that word.
@@ -109,6 +114,13 @@ struct Streamed {
     double bytes_h2d = 0, bytes_d2h = 0, seconds = 0;
     std::vector<hipEvent_t> tl_events;  // 4 per chunk when timing is on: H2D begin/end, D2H begin/end
     std::vector<float> timeline;        // ms since the first H2D began
+    // Host arrays that are not pinned (ordinary CPU tensors) go up through pinned bounce buffers that
+    // host threads fill while earlier chunks are on the link; see streamed_enqueue_impl.
+    void* bounce[4][kBounce] = {};
+    size_t bounce_cap[4] = {0, 0, 0, 0};   // bytes of each of the kBounce buffers of an array
+    std::unique_ptr<CopyPool> pool;
+    int bounce_threads = 4;   // RT_STREAM_BOUNCE_THREADS in the environment overrides; 0 leaves such copies to the runtime
+    uint64_t paced_calls = 0, bounced_bytes = 0;
 };
 
 }  // namespace
@@ -725,9 +737,9 @@ int rt_destroy(rt_handle* h) {
     }
     Streamed& st = h->st;
     for (int a = 0; a < 4; ++a)
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < kStageBufs; ++b)
             if (st.stage[a][b].ptr) (void)hipFree(st.stage[a][b].ptr);
-    for (int b = 0; b < 2; ++b) {
+    for (int b = 0; b < kStageBufs; ++b) {
         if (st.h2d_done[b]) (void)hipEventDestroy(st.h2d_done[b]);
         if (st.comp_done[b]) (void)hipEventDestroy(st.comp_done[b]);
         if (st.d2h_done[b]) (void)hipEventDestroy(st.d2h_done[b]);
@@ -736,6 +748,10 @@ int rt_destroy(rt_handle* h) {
         if (r.dev.ptr) (void)hipFree(r.dev.ptr);
         if (r.host) (void)hipHostFree(r.host);
     }
+    st.pool.reset();  // joins the copy threads
+    for (int a = 0; a < 4; ++a)
+        for (int k = 0; k < kBounce; ++k)
+            if (st.bounce[a][k]) (void)hipHostFree(st.bounce[a][k]);
     if (st.ticket_word) (void)hipHostFree((void*)st.ticket_word);
     for (hipEvent_t e : st.tl_events) (void)hipEventDestroy(e);
     if (st.start) (void)hipEventDestroy(st.start);
@@ -971,9 +987,10 @@ static int streamed_init(rt_handle* h) {
     // memory, say) can be repeated without leaking what the first attempt created.
     for (hipStream_t* s : {&st.h2d, &st.comp, &st.d2h})
         if (!*s) HIP_TRY(hipStreamCreateWithFlags(s, hipStreamNonBlocking));
-    for (hipEvent_t* e : {&st.start, &st.h2d_done[0], &st.h2d_done[1], &st.comp_done[0], &st.comp_done[1],
-                          &st.d2h_done[0], &st.d2h_done[1]})
-        if (!*e) HIP_TRY(hipEventCreateWithFlags(e, hipEventDisableTiming));
+    if (!st.start) HIP_TRY(hipEventCreateWithFlags(&st.start, hipEventDisableTiming));
+    for (int b = 0; b < kStageBufs; ++b)
+        for (hipEvent_t* e : {&st.h2d_done[b], &st.comp_done[b], &st.d2h_done[b]})
+            if (!*e) HIP_TRY(hipEventCreateWithFlags(e, hipEventDisableTiming));
     // Table memory for the calls in flight is set aside now: allocating (device or pinned
     // host memory) while the copy pipeline runs stalls the copies for tens of milliseconds.
     if (st.ring.size() < kTablePool) st.ring.resize(kTablePool);
@@ -999,6 +1016,7 @@ static int streamed_init(rt_handle* h) {
         const long v = atol(e);
         if (v > 0) st.batch_chunks = (uint64_t)v;
     }
+    if (const char* e = getenv("RT_STREAM_BOUNCE_THREADS")) st.bounce_threads = (int)std::min(64l, std::max(0l, atol(e)));
     st.ready = true;
     return RT_OK;
 }
@@ -1107,6 +1125,32 @@ static int streamed_wait(rt_handle* h) {
     return RT_OK;
 }
 
+// True for host memory the runtime has pinned (hipHostMalloc, torch's pin_memory): copies from it
+// are asynchronous.  Anything else -- an ordinary CPU tensor -- the runtime would stage through
+// its own buffers while the calling thread waits.
+static bool is_pinned_host(const void* p) {
+    hipPointerAttribute_t attr;
+    memset(&attr, 0, sizeof(attr));
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void)hipGetLastError();  // unknown pointer: the error is the answer, not a failure
+        return false;
+    }
+    return attr.type == hipMemoryTypeHost;
+}
+
+// Waits for the copies of every chunk whose fill has been submitted when a call leaves early: the
+// workers read the caller's arrays and the groups live on the caller's stack.
+namespace {
+struct FillGuard {
+    CopyPool* pool = nullptr;
+    CopyPool::Group* groups = nullptr;
+    size_t submitted = 0;
+    ~FillGuard() {
+        for (size_t i = 0; pool && i < submitted; ++i) pool->wait(&groups[i]);
+    }
+};
+}  // namespace
+
 // Validates and enqueues the whole pipeline of one call; does not wait for it.
 static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
                             uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems,
@@ -1149,7 +1193,7 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
     for (const auto& c : chunks)
         if (!c.empty()) max_used = std::max(max_used, align_up(c.back().stage_off + c.back().count, kVec));
     for (int a = 0; a < 4; ++a)
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < kStageBufs; ++b)
             if (stage_esize[a]) {
                 // sized for fp32 (or wider) so that the common dtype changes never reallocate
                 const size_t want = max_used * std::max(4, stage_esize[a]);
@@ -1161,6 +1205,52 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
                 if (rc != RT_OK) return rc;
             }
 
+    // ---- host arrays that are not pinned.  Their uploads go through pinned bounce buffers: host
+    //      threads copy chunk c+1 and c+2 into them while chunk c is on the link, and the host hands
+    //      the pipeline one chunk at a time (at most kPacedInFlight on the streams, see below)
+    //      instead of queuing everything up front.  Left to the runtime, such a copy is staged
+    //      inside hipMemcpyAsync while the calling thread waits, and nothing else gets queued.
+    std::vector<uint8_t> unpinned(n, 0);  // bit a: array a of the tensor is host memory that is not pinned
+    bool paced = false;
+    if (st.bounce_threads > 0)
+        for (uint32_t i = 0; i < n; ++i) {
+            const rt_tensor_desc& d = descs[i];
+            if (d.numel == 0) continue;
+            const void* host[4] = {d.p, d.g, d.m, d.v};
+            for (int a = 0; a < 4; ++a)
+                if ((d.host_mask & (1u << a)) && !is_pinned_host(host[a])) unpinned[i] |= (uint8_t)(1u << a);
+            paced |= unpinned[i] != 0;
+        }
+    if (paced) {
+        // the bounce buffers and the chunk counter are shared with earlier calls: let those finish
+        if (st.pending) {
+            rc = streamed_wait(h);
+            if (rc != RT_OK) return rc;
+        }
+        if (!st.pool) st.pool.reset(new CopyPool((unsigned)st.bounce_threads));
+        bool need[4] = {false, false, false, false};
+        for (uint32_t i = 0; i < n; ++i)
+            for (int a = 0; a < 4; ++a) need[a] |= (unpinned[i] >> a) & 1;
+        for (int a = 0; a < 4; ++a) {
+            const size_t want = max_used * (size_t)stage_esize[a];
+            if (!need[a] || want <= st.bounce_cap[a]) continue;
+            for (int k = 0; k < kBounce; ++k) {
+                if (st.bounce[a][k]) HIP_TRY(hipHostFree(st.bounce[a][k]));
+                st.bounce[a][k] = nullptr;
+            }
+            st.bounce_cap[a] = 0;
+            for (int k = 0; k < kBounce; ++k) {
+                hipError_t e = hipHostMalloc(&st.bounce[a][k], want, hipHostMallocDefault);
+                if (e != hipSuccess) {
+                    st.bounce[a][k] = nullptr;
+                    return fail(RT_ENOMEM, "hipHostMalloc(%zu) for a bounce buffer failed: %s", want, hipGetErrorString(e));
+                }
+            }
+            st.bounce_cap[a] = want;
+        }
+        ++st.paced_calls;
+    }
+
     // ---- descriptors of every piece (pointers into staging for host-resident arrays), and the
     //      table images of all chunks, uploaded in one copy before the pipeline starts
     std::vector<std::vector<rt_tensor_desc>> pieces(chunks.size());
@@ -1168,7 +1258,7 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
     std::vector<size_t> plan_off(chunks.size());
     std::vector<uint8_t> blob;
     for (size_t c = 0; c < chunks.size(); ++c) {
-        const int b = (int)((st.seq + c) & 1);
+        const int b = (int)((st.seq + c) % kStageBufs);
         for (const Segment& s : chunks[c]) {
             const rt_tensor_desc& d = descs[s.tensor];
             rt_tensor_desc q = d;
@@ -1254,21 +1344,58 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
         }
     }
     const uint64_t batch = st.batch_chunks;
+    std::unique_ptr<CopyPool::Group[]> fills(paced ? new CopyPool::Group[chunks.size()] : nullptr);
+    FillGuard guard;
+    guard.pool = st.pool.get();
+    guard.groups = fills.get();
+    // Chunk k may be copied into its bounce buffers once chunk k - kBounce has left them, which is
+    // known when that chunk's D2H has been published.
+    auto submit_fills_through = [&](size_t last) {
+        for (; guard.submitted <= last && guard.submitted < chunks.size(); ++guard.submitted) {
+            const size_t k = guard.submitted;
+            const int slot = (int)((st.seq + k) % kBounce);
+            for (const Segment& s : chunks[k]) {
+                const rt_tensor_desc& d = descs[s.tensor];
+                const uint8_t up = unpinned[s.tensor];
+                if (!up) continue;
+                const int es[4] = {dtype_size(d.p_dtype), dtype_size(d.g_dtype), dtype_size(d.m_dtype),
+                                   dtype_size(d.v_dtype)};
+                const void* host[4] = {d.p, d.g, d.m, d.v};
+                for (int a = 0; a < 4; ++a)
+                    if (up & (1u << a)) {
+                        st.pool->submit(&fills[k], (uint8_t*)st.bounce[a][slot] + s.stage_off * es[a],
+                                        (const uint8_t*)host[a] + s.start * es[a], s.count * es[a]);
+                        st.bounced_bytes += s.count * es[a];
+                    }
+            }
+        }
+    };
     for (size_t c = 0; c < chunks.size(); ++c) {
-        const int b = (int)((st.seq + c) & 1);
+        const int b = (int)((st.seq + c) % kStageBufs);
         const auto& segs = chunks[c];
+        if (paced) {
+            // The host feeds the pipeline: chunk c goes onto the streams when chunk c - kPacedInFlight
+            // has come back (with a third chunk queued while two are on the streams the copies were
+            // measured at a third of their rate, also with three staging buffers per array),
+            // and when the host threads have filled its bounce buffers.  Every wait is a sleep on a
+            // word of pinned memory or on the pool's condition variable, never inside the runtime.
+            if (c >= kPacedInFlight && !sleep_until_word(st.ticket_word + 1, st.seq + c - kPacedInFlight + 1))
+                HIP_TRY(hipStreamSynchronize(st.d2h));  // stalled: block, and surface a device error
+            submit_fills_through(c + kBounce - kPacedInFlight);
+            st.pool->wait(&fills[c]);
+        }
         // A long call is queued in batches, and the pipeline drains between them.  With a few
         // hundred chunks waiting on the streams at once the copies of this pipeline were measured
         // at well under half their rate, and queuing more while the streams are busy costs about
         // as much; a drain costs one pipeline fill (about two chunk times) per batch.
-        if (c > 0 && c % batch == 0) {
+        if (!paced && c > 0 && c % batch == 0) {
             hipLaunchKernelGGL(publish_ticket_kernel, dim3(1), dim3(1), 0, st.d2h,
                                (uint64_t)(st.ticket_word + 1), st.seq + c);
             HIP_TRY(hipGetLastError());
             if (!sleep_until_word(st.ticket_word + 1, st.seq + c))
                 HIP_TRY(hipStreamSynchronize(st.d2h));  // stalled: block, and surface a device error
         }
-        // H2D: the buffer is free once the D2H of the chunk two back has finished
+        // H2D: the buffer is free once the D2H of the chunk that used it last has finished
         if (st.used_buf[b]) HIP_TRY(hipStreamWaitEvent(st.h2d, st.d2h_done[b], 0));
         if (trace) HIP_TRY(hipEventRecord(st.tl_events[4 * c + 0], st.h2d));
         for (size_t k = 0; k < segs.size(); ++k) {
@@ -1281,8 +1408,10 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
             for (int a = 0; a < 4; ++a) {
                 if (!(d.host_mask & (1u << a))) continue;
                 const size_t bytes = s.count * es[a];
-                HIP_TRY(hipMemcpyAsync(dev[a], (const uint8_t*)host[a] + s.start * es[a], bytes,
-                                       hipMemcpyHostToDevice, st.h2d));
+                const uint8_t* src = (unpinned[s.tensor] & (1u << a))
+                                         ? (const uint8_t*)st.bounce[a][(st.seq + c) % kBounce] + s.stage_off * es[a]
+                                         : (const uint8_t*)host[a] + s.start * es[a];
+                HIP_TRY(hipMemcpyAsync(dev[a], src, bytes, hipMemcpyHostToDevice, st.h2d));
                 st.bytes_h2d += (double)bytes;
             }
         }
@@ -1316,6 +1445,11 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
         if (trace) HIP_TRY(hipEventRecord(st.tl_events[4 * c + 3], st.d2h));
         HIP_TRY(hipEventRecord(st.d2h_done[b], st.d2h));
         st.used_buf[b] = true;
+        if (paced) {
+            hipLaunchKernelGGL(publish_ticket_kernel, dim3(1), dim3(1), 0, st.d2h, (uint64_t)(st.ticket_word + 1),
+                               st.seq + c + 1);
+            HIP_TRY(hipGetLastError());
+        }
     }
     st.seq += chunks.size();
     tab.ticket = st.tickets_issued + 1;
@@ -1348,7 +1482,7 @@ static int streamed_enqueue(rt_handle* h, const rt_tensor_desc* descs, uint32_t 
         (void)hipStreamSynchronize(st.h2d);
         (void)hipStreamSynchronize(st.comp);
         (void)hipStreamSynchronize(st.d2h);
-        st.used_buf[0] = st.used_buf[1] = false;
+        for (bool& u : st.used_buf) u = false;
         st.pending = false;
         for (auto& r : st.ring) r.in_flight = false;
         memcpy(g_err, saved, sizeof(saved));
@@ -1531,6 +1665,13 @@ int rt_streamed_stats(rt_handle* h, double out[3]) {
     out[0] = h->st.bytes_h2d;
     out[1] = h->st.bytes_d2h;
     out[2] = h->st.seconds;
+    return RT_OK;
+}
+
+int rt_streamed_bounce_stats(rt_handle* h, uint64_t out[2]) {
+    if (!h || !out) return fail(RT_EINVAL, "NULL argument");
+    out[0] = h->st.paced_calls;
+    out[1] = h->st.bounced_bytes;
     return RT_OK;
 }
 

@@ -95,6 +95,38 @@ def test_streamed_mixed_residency_and_dtypes(handle):
     np.testing.assert_array_equal(e1.v.numpy().view(np.uint32), b[2].view(np.uint32))
 
 
+@pytest.mark.parametrize("chunk_elems", [64, 4096, 65_536])
+def test_unpinned_gradients_go_up_through_bounce_buffers(handle, chunk_elems):
+    """The reference's offload flow leaves the gradients in ordinary CPU memory (linear.py:416-427):
+    host threads copy them into pinned bounce buffers chunk by chunk.  More chunks than bounce
+    buffers, pinned and unpinned gradients in one call, two calls in a row (the buffer index
+    runs on across calls), and an unpinned parameter next to pinned states."""
+    lens = [30_011, 8, 0, 4096, 100_000, 5, 8193]
+    before = handle.streamed_bounce_stats()
+    state = []
+    for i, n in enumerate(lens):
+        p, g, m, v = oracle.synth_inputs(n, 500 + i)
+        state.append([p, g, m, v, host16(p, pin=(i != 4)), host16(m), host16(v)])
+    expect_bytes = 0
+    for step in (7, 8):
+        sc, sco = F.make_scalars(step=step, **HP0), oracle.scalars_from_hparams(step=step, **HP0)
+        entries = []
+        for i, (p, g, m, v, P, M, V) in enumerate(state):
+            unpinned = i % 3 != 1
+            G = host16(g, pin=not unpinned)
+            assert G.is_pinned() != unpinned or len(g) == 0
+            entries.append(F.Entry(p=P, g=G, m=M, v=V, step=step, scalars_idx=0, tensor_id=i))
+            expect_bytes += 2 * len(g) * unpinned + 2 * len(p) * (i == 4)
+        F.step_streamed(handle, entries, [sc], seed=31, explicit_noise=False, chunk_elems=chunk_elems)
+        for i, (p, g, m, v, P, M, V) in enumerate(state):
+            oracle.step_tensor(p, g, m, v, sco, seed=31, step=step, tensor_id=i)
+            for name, t, a in zip("pmv", (P, M, V), (p, m, v)):
+                np.testing.assert_array_equal(bits16(t), a, err_msg=f"step {step} chunk {chunk_elems} tensor {i} {name}")
+    after = handle.streamed_bounce_stats()
+    assert after["calls"] - before["calls"] == 2
+    assert after["bytes"] - before["bytes"] == expect_bytes
+
+
 def test_streamed_and_resident_agree_bit_for_bit(handle):
     n = 300_000
     p, g, m, v = oracle.synth_inputs(n, 95)
