@@ -29,8 +29,8 @@ ema~N(0,1e-4), ema_squared=N(0,1e-3)^2, stored bf16):
   mixed     Llama-3-8B shapes; bf16 p and ema, fp32 ema_squared, fp32 grads scaled
             by 1024 and unscaled in-kernel, global-norm clip to 1.0
   central   the default set with centralization=1.0 (adamw.py:179-184): one row-mean
-            pass per matrix (2 B per element read) and the update through the
-            kernel that subtracts the means (14 B per element + 4 B per row)
+            pass per tensor (2 B per element read) and the update through the fast
+            kernel's instance that subtracts the means (14 B per element + 4 B per row)
   streamed  Llama-3-8B shapes with p/ema/ema_squared in pinned host memory,
             bf16 grads on the GPU, 256 MB chunks (--stream-gb bounds the host set)
   hooked    the same set, but each tensor is updated by AdamW.step_param() as a
@@ -310,7 +310,7 @@ def run_resident(wl, args, steps, warmup, *, full):
                 "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic[0] if traffic else None,
                 "traffic_source": (f"not measured in this run: rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of an earlier "
                                    f"run, {traffic[1]}") if traffic else None,
-                "kernel": {"mixed": "sr_adamw_fast_wide_kernel", "central": "sr_adamw_generic_kernel"}.get(wl, "sr_adamw_fast_kernel"),
+                "kernel": {"mixed": "sr_adamw_fast_wide_kernel", "central": "sr_adamw_fast_kernel (centralizing instance)"}.get(wl, "sr_adamw_fast_kernel"),
                 "kernel_ms": k_ms, "kernel_launches_timed": len(ks), "algorithmic_bytes_per_launch": upd_bytes}
     out = {"ms_per_step": ms_per_step, "elements_per_s": total / (ms_per_step * 1e-3),
            "achieved_GBps_wall": STEP_BYTES[wl] * total / (ms_per_step * 1e-3) / 1e9,

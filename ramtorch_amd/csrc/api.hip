@@ -135,6 +135,7 @@ struct Batch {            // tensors of one dtype combination inside a table ima
     uint32_t first_range, n_ranges, n_units;   // fast kernel: entries of the range list, fast units
     uint32_t first_piece, n_pieces;            // pieces served by the fast kernel's first workgroups
     uint32_t first_generic, n_generic;         // chunk range of the generic kernel
+    uint32_t first_cen_range, n_cen_ranges, n_cen_units;  // the same lists for tensors with centralization
 };
 
 struct Plan {
@@ -237,7 +238,8 @@ using MultiKernel = void (*)(const LaunchArgs);
 
 struct KernelPair {
     MultiKernel fast;     // whole fast units of aligned tensors, plus (16-bit layouts, Philox) their pieces
-    MultiKernel generic;  // unaligned tensors, debug outputs, centralization, leftovers without a piece path
+    MultiKernel generic;  // unaligned tensors, debug outputs, leftovers without a piece path, rows shorter than 8
+    MultiKernel fast_cen; // whole fast units of aligned tensors with centralization (16-bit layouts, Philox), or NULL
 };
 
 template <int P, int G, int M, int V>
@@ -247,14 +249,15 @@ static KernelPair pick_noise(int noise) {
     if constexpr (wide) {
         if (noise == RT_NOISE_EXPLICIT)
             return {sr_adamw_fast_wide_kernel<P, G, M, V, RT_NOISE_EXPLICIT>,
-                    sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_EXPLICIT>};
+                    sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_EXPLICIT>, nullptr};
         return {sr_adamw_fast_wide_kernel<P, G, M, V, RT_NOISE_PHILOX>,
-                sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_PHILOX>};
+                sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_PHILOX>, nullptr};
     } else {
         if (noise == RT_NOISE_EXPLICIT)
             return {sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_EXPLICIT>,
-                    sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_EXPLICIT>};
-        return {sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_PHILOX>, sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_PHILOX>};
+                    sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_EXPLICIT>, nullptr};
+        return {sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_PHILOX>, sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_PHILOX>,
+                sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_PHILOX, true>};
     }
 }
 // State dtype pairs the templated kernels are instantiated for: every bf16 / fp32 mix, and both fp16.
@@ -456,12 +459,31 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
         b.n_ranges = (uint32_t)ranges.size() - b.first_range;
         b.n_units = units;
         b.n_pieces = (uint32_t)pieces.size() - b.first_piece;
+        // Tensors with centralization that are otherwise plain: their whole units go to the fast
+        // kernel's centralizing variant (16-bit layouts with Philox noise have one), the rest of them
+        // to the generic kernel.  A lane's 8 elements must lie in at most two rows.
+        auto cen_plain = [&](const DevTensor& t) {
+            return has_pieces && (t.flags & kFlagAligned) && (t.dp | t.dm | t.dv) == 0 && t.row_mean != 0 &&
+                   t.row_len >= (uint64_t)kVec && t.row_len < (1ull << 31);
+        };
+        b.first_cen_range = (uint32_t)ranges.size();
+        uint32_t cen_units = 0;
+        for (size_t k = k0; k < k1; ++k) {
+            const DevTensor& t = tens[k];
+            if (!cen_plain(t) || t.numel < unit) continue;
+            ranges.push_back(cen_units);
+            fast_tens.push_back(t);
+            cen_units += (uint32_t)(t.numel / unit);
+        }
+        b.n_cen_ranges = (uint32_t)ranges.size() - b.first_cen_range;
+        b.n_cen_units = cen_units;
         b.first_generic = (uint32_t)chunks.size();
         for (size_t k = k0; k < k1; ++k) {
             const DevTensor& t = tens[k];
             const uint32_t nc = (uint32_t)((t.numel + kChunkElems - 1) / kChunkElems);
             uint32_t j0 = 0;
             if (plain(t)) j0 = has_pieces ? nc : (uint32_t)(t.numel / kChunkElems);
+            if (cen_plain(t)) j0 = (uint32_t)(t.numel / kChunkElems);
             for (uint32_t j = j0; j < nc; ++j) chunks.push_back(ChunkRef{(uint32_t)k, j});
         }
         b.n_generic = (uint32_t)chunks.size() - b.first_generic;
@@ -585,6 +607,15 @@ static int enqueue_kernels(const Plan& plan, const uint8_t* base, uint64_t seed,
         if (grid > kMaxGrid || b.n_generic > kMaxGrid) return fail(RT_EUNSUPPORTED, "too many workgroups in one launch");
         if (grid) launches.push_back(Launch{k.fast, (uint32_t)grid, a});
         if (b.n_generic) launches.push_back(Launch{k.generic, b.n_generic, a});
+        if (b.n_cen_units) {
+            if (!k.fast_cen) return fail(RT_EHIP, "internal: centralized units without a kernel for them");
+            LaunchArgs c = a;
+            c.first = (const uint32_t*)(base + plan.off_ranges) + b.first_cen_range;
+            c.fast_tensors = (const DevTensor*)(base + plan.off_fast_tensors) + b.first_cen_range;
+            c.n_ranges = b.n_cen_ranges;
+            c.n_pieces = c.n_piece_wgs = c.piece_rate = 0;
+            launches.push_back(Launch{k.fast_cen, b.n_cen_units, c});
+        }
     }
     for (size_t i = 0; i < launches.size(); ++i) {
         const Launch& l = launches[i];

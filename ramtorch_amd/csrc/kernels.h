@@ -438,7 +438,10 @@ __device__ __forceinline__ void piece_body(const LaunchArgs& a, uint32_t q) {
 // Everything is inlined and lives in registers: a stack frame here would turn
 // into scratch-memory traffic on every workgroup.
 // ---------------------------------------------------------------------------
-template <int PDT, int GDT, int MDT, int VDT, int NOISE>
+// CEN: the tensors of the launch have their gradients centralized (adamw.py:179-184): fl(mean(row) * c)
+// is subtracted from every gradient element before the update.  Rows are at least 8 elements long
+// (shorter ones take the generic kernel), so a lane's 8 elements lie in at most two rows.
+template <int PDT, int GDT, int MDT, int VDT, int NOISE, bool CEN = false>
 __global__ __launch_bounds__(kThreads) void sr_adamw_fast_kernel(const LaunchArgs a) {
     if (a.skip != nullptr && load_const(a.skip) != 0u) return;
     // Piece workgroups are spread evenly among the unit workgroups: of the first b workgroups,
@@ -474,8 +477,11 @@ __global__ __launch_bounds__(kThreads) void sr_adamw_fast_kernel(const LaunchArg
         Raw8<MDT> m;
         Raw8<VDT> v;
         u32x4 zp, zm, zv;
+        float mean0, mean1;  // CEN: means of the row of the first element and of the row after it
+        uint32_t rem;        // CEN: position of the first element inside its row
     };
-    auto fetch = [&](uint64_t i) {
+    const uint32_t row_len = (uint32_t)t.row_len;  // CEN launches: 8 <= row_len < 2^31
+    auto fetch = [&](uint64_t i, uint64_t row, uint32_t rem) {
         In r;
         r.p = load_raw<PDT>(tp, i);
         r.g = load_raw<GDT>(tg, i);
@@ -486,6 +492,11 @@ __global__ __launch_bounds__(kThreads) void sr_adamw_fast_kernel(const LaunchArg
             if constexpr (MDT == RT_DT_BF16) r.zm = ldg128(tnm + i * 2);
             if constexpr (VDT == RT_DT_BF16) r.zv = ldg128(tnv + i * 2);
         }
+        if constexpr (CEN) {
+            r.rem = rem;
+            r.mean0 = ldg32f(t.row_mean + row * 4);
+            r.mean1 = rem + (kVec - 1) >= row_len ? ldg32f(t.row_mean + row * 4 + 4) : 0.0f;
+        }
         return r;
     };
     // A wave walks its own contiguous quarter of the unit (4 x 1 KB per array)
@@ -495,12 +506,29 @@ __global__ __launch_bounds__(kThreads) void sr_adamw_fast_kernel(const LaunchArg
     constexpr uint64_t kStep = 64 * kVec;
     const uint64_t i0 = (uint64_t)unit_in_tensor * kFastUnitElems +
                         (uint64_t)(threadIdx.x >> 6) * (kStep * kItersPerChunk) + (uint64_t)(threadIdx.x & 63u) * kVec;
-    In cur = fetch(i0);
+    // CEN: one 64-bit division finds the row of the lane's first element; from vector to vector the
+    // position advances by kStep elements, which a 32-bit division turns into rows.
+    uint64_t row = 0;
+    uint32_t rem = 0;
+    if constexpr (CEN) {
+        const uint64_t e0 = (t.block_base << 3) + i0;
+        row = e0 / row_len;
+        rem = (uint32_t)(e0 - row * row_len);
+    }
+    In cur = fetch(i0, row, rem);
 #pragma unroll
     for (int it = 0; it < kItersPerChunk; ++it) {
         const uint64_t i = i0 + (uint64_t)it * kStep;
         In nxt;
-        if (it + 1 < kItersPerChunk) nxt = fetch(i + kStep);
+        if (it + 1 < kItersPerChunk) {
+            if constexpr (CEN) {
+                const uint32_t ahead = rem + (uint32_t)kStep;  // < 2^31 + 512
+                const uint32_t q = ahead / row_len;
+                row += q;
+                rem = ahead - q * row_len;
+            }
+            nxt = fetch(i + kStep, row, rem);
+        }
 
         float p[8], g[8], m[8], v[8];
         decode<PDT>(cur.p, p);
@@ -510,6 +538,12 @@ __global__ __launch_bounds__(kThreads) void sr_adamw_fast_kernel(const LaunchArg
         u32x4 zp = cur.zp, zm = cur.zm, zv = cur.zv;
         if constexpr (NOISE == RT_NOISE_PHILOX) philox_noise3<PDT, MDT, VDT>(t, c, i, zp, zm, zv);
         scale_grads(g, c);
+        if constexpr (CEN) {
+            // grad.sub_(mean.mul_(c)): the product is rounded, then subtracted
+            const float mc0 = cur.mean0 * c.s.centralization, mc1 = cur.mean1 * c.s.centralization;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) g[j] = g[j] - (cur.rem + (uint32_t)j < row_len ? mc0 : mc1);
+        }
         update_n<8>(p, g, m, v, c.s);
         store_out<PDT>(tp, i, p, zp);
         store_out<MDT>(tm, i, m, zm);

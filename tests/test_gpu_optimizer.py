@@ -325,7 +325,8 @@ def test_optimizer_with_loss_scale_and_max_grad_norm():
     assert opt.last_grad_norm.view(torch.int32)[2].item() == 1
 
 
-@pytest.mark.parametrize("shape", [(37, 24), (4, 3, 10), (129,), ()])
+@pytest.mark.parametrize("shape", [(37, 24), (4, 3, 10), (129,), (), (64, 300), (3000, 8), (5, 4099), (16, 1024, 3),
+                                   (20_000,), (4, 8192), (2500, 7)])
 def test_centralization(shape):
     n = int(np.prod(shape)) if len(shape) else 1
     p, g, _, _ = oracle.synth_inputs(n, 800)
@@ -350,6 +351,26 @@ def test_centralization(shape):
     gt = gt - gt.mean(dim=tuple(range(1, gt.dim())), keepdim=True) * 0.5
     np.testing.assert_allclose(g32.reshape(shape), gt.cpu().numpy(), rtol=1e-5, atol=1e-9)
     h.close()
+
+
+@pytest.mark.parametrize("shape", [(64, 300), (3, 70_001), (9000, 12)])
+def test_centralization_in_pieces_equals_whole(shape):
+    """Host-resident states: the tensor is updated in staged pieces that start in the middle of rows
+    (and of the tensor); whole units of a piece take the fast kernel's centralizing variant, the
+    rest the generic kernel.  Same bits as the resident step."""
+    n = int(np.prod(shape))
+    p, g, _, _ = oracle.synth_inputs(n, 810)
+    out = []
+    for storage, extra in (("cuda", {}), ("cpu", dict(stream_chunk_bytes=2 * 10_000))):
+        P = torch.nn.Parameter(dev16(p).view(shape))
+        P.grad = dev16(g).view(shape)
+        opt = ramtorch_amd.AdamW([P], storage_device=storage, seed=3, centralization=0.25, **extra, **HP0)
+        for _ in range(2):
+            opt.step()
+        torch.cuda.synchronize()
+        out.append((bits16(P), bits16(opt.state[P]["ema"]), bits16(opt.state[P]["ema_squared"])))
+    for a, b in zip(*out):
+        np.testing.assert_array_equal(a, b)
 
 
 def test_copy_stochastic():
