@@ -66,6 +66,7 @@ OFFLINE_TRAFFIC = {
     "mixed": (160_597_606_615, _TRAFFIC_FILE),      # the update launch; its norm pass fetches 32 120 545 889 B more
     "small": (1_090_935_301, _TRAFFIC_FILE),
     "cfg0": (335_774_529, _TRAFFIC_FILE),
+    "central": (112_473_148_416 + 3_860_685, _TRAFFIC_FILE),   # centralizing fast instance + generic kernel for the norm vectors
 }
 HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
 METRIC = "SR-AdamW step: params/sec + achieved HBM GB/s (% of peak), 8B bf16 set, 1 GPU"
