@@ -555,19 +555,7 @@ class AdamW(Optimizer):
                     if not g.is_cuda:
                         g = g.to(f"cuda:{dev}", non_blocking=True)
                         e.g = g
-                    # adamw.py:179-184: mean over every dim but the first (all dims for 0-d / 1-d)
-                    rows = g.shape[0] if g.dim() >= 2 else 1
-                    row_len = g.numel() // rows if rows else 0
-                    if g.numel():
-                        if getattr(self, "noise_source", "philox") == "reference" and inv_loss_scale == 1.0:
-                            # the verification mode reproduces the reference bit for bit: the means come
-                            # from the very call the reference makes (a sum's bits depend on its order)
-                            g32 = g.to(torch.float32)
-                            e.row_mean = g32.mean(dim=tuple(range(1, g32.dim())), keepdim=True).reshape(-1).contiguous()
-                        else:
-                            with torch.cuda.device(dev):
-                                e.row_mean = F.row_means(_handle(dev), g, rows, row_len, inv_loss_scale)
-                        e.row_len = row_len
+                    e.row_mean, e.row_len = self._row_means(g, dev, inv_loss_scale)
                 if noise is not None and p in noise:
                     e.noise = tuple(noise[p])
                 if debug_out is not None and p in debug_out:
@@ -769,6 +757,21 @@ class AdamW(Optimizer):
                 self.step_param(param, grad if grad is not None else param.grad)
         return hook
 
+    def _row_means(self, g: torch.Tensor, dev: int, inv_loss_scale: float):
+        """(fp32 row means of the GPU gradient ``g``, row length) for centralization, adamw.py:179-184:
+        the mean over every dim but the first (over all of them for 0-d / 1-d)."""
+        rows = g.shape[0] if g.dim() >= 2 else 1
+        row_len = g.numel() // rows if rows else 0
+        if not g.numel():
+            return None, 0
+        if getattr(self, "noise_source", "philox") == "reference" and inv_loss_scale == 1.0:
+            # the verification mode reproduces the reference bit for bit: the means come
+            # from the very call the reference makes (a sum's bits depend on its order)
+            g32 = g.to(torch.float32)
+            return g32.mean(dim=tuple(range(1, g32.dim())), keepdim=True).reshape(-1).contiguous(), row_len
+        with torch.cuda.device(dev):
+            return F.row_means(_handle(dev), g, rows, row_len, inv_loss_scale), row_len
+
     def step_param(self, p: torch.Tensor, grad: Optional[torch.Tensor] = None) -> None:
         """Update one parameter now, without waiting: same arithmetic, same noise and same
         ``state["step"]`` bookkeeping as ``step()`` would apply to it.  The update is queued
@@ -793,8 +796,6 @@ class AdamW(Optimizer):
             raise ValueError("step_param: tensor is not a parameter of this optimizer")
         gi, k = pos
         group = self.param_groups[gi]
-        if group["centralization"] != 0:
-            raise NotImplementedError("step_param with centralization")
         r = recs[gi][k]
         state = r.state
         if (state.get("ema") is not r.m or state.get("ema_squared") is not r.v or p.data_ptr() != r.p_ptr
@@ -815,9 +816,12 @@ class AdamW(Optimizer):
             step = state["step"] + 1
             state["step"] = step
             inv_loss_scale = 1.0 / self.loss_scale if self.loss_scale != 1.0 else 1.0
+            cen = group["centralization"]
             sc = [F.make_scalars(group["lr"], tuple(group["betas"]), group["eps"], group["weight_decay"], step,
-                                 inv_loss_scale=inv_loss_scale)]
+                                 centralization=cen, inv_loss_scale=inv_loss_scale)]
             e = F.Entry(p=p.data, g=g, m=r.m, v=r.v, step=step, scalars_idx=0, tensor_id=r.tensor_id)
+            if cen != 0:
+                e.row_mean, e.row_len = self._row_means(g, dev, inv_loss_scale)
             h = _handle(dev)
             with torch.cuda.device(dev):
                 if e.p.is_cuda and e.m.is_cuda and e.v.is_cuda:
@@ -855,8 +859,8 @@ class AdamW(Optimizer):
                 else:
                     sl = slice(used, used + take)
                     piece = F.Entry(p=e.p.view(-1)[sl], g=e.g.view(-1)[sl], m=e.m.view(-1)[sl], v=e.v.view(-1)[sl],
-                                    step=e.step, scalars_idx=0, tensor_id=e.tensor_id,
-                                    elem_offset=e.elem_offset + used, keep=[e])
+                                    step=e.step, scalars_idx=0, tensor_id=e.tensor_id, row_mean=e.row_mean,
+                                    row_len=e.row_len, elem_offset=e.elem_offset + used, keep=[e])
                 piece.scalars_idx = len(scalars)
                 scalars.append(sc)
                 entries.append(piece)

@@ -259,6 +259,34 @@ def test_post_accumulate_hook_updates_from_the_gpu_gradient():
         np.testing.assert_array_equal(bits16(p), refs[i][0], err_msg=f"step 3 param {i}")
 
 
+def test_step_param_with_centralization_equals_step():
+    """Updates handed over tensor by tensor (the hook of ramtorch.Linear) with gradient centralization
+    (adamw.py:179-184): the row means are taken from the whole gradient, the update then goes in
+    staged pieces that start in the middle of rows.  Same bits as step() on the same data."""
+    shapes = [(64, 300), (5, 4099), (129,), (9000, 12)]
+    out = []
+    for early in (False, True):
+        ps, gs, _ = _offload_params(shapes, 1250)
+        q = torch.nn.Parameter(dev16(gs[1]).view(shapes[1]).clone())   # a GPU-resident parameter as well
+        opt = ramtorch_amd.AdamW(ps + [q], seed=9, centralization=0.5, stream_chunk_bytes=2 * 10_000, **HP0)
+        for k in ("ema", "ema_squared"):
+            opt.state[q][k] = opt.state[q][k].cuda()
+        for _ in range(2):
+            grads = [dev16(g).view(shp) for g, shp in zip(gs, shapes)] + [dev16(gs[3])[:q.numel()].view(q.shape)]
+            if early:
+                for p, g in zip(ps + [q], grads):
+                    opt.step_param(p, g)
+                opt.step()
+            else:
+                opt.step(grads=dict(zip(ps + [q], grads)))
+        torch.cuda.synchronize()
+        out.append([(bits16(p), bits16(opt.state[p]["ema"]), bits16(opt.state[p]["ema_squared"])) for p in ps + [q]])
+        assert all(opt.state[p]["step"] == 2 for p in ps + [q])
+    for a, b in zip(*out):
+        for x, y in zip(a, b):
+            np.testing.assert_array_equal(x, y)
+
+
 def test_step_param_mixes_with_step_and_rejects_double_use():
     ps, gs, refs = _offload_params([(3000,), (5000,)], 1300)
     gpu_p, gpu_g, _, _ = oracle.synth_inputs(7000, 1310)
