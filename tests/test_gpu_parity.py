@@ -434,3 +434,61 @@ def test_random_cases_match_the_oracle(handle):
                   debug=bool(rng.random() < 0.5))
         got, want, dbg, pre = run_both(handle, conv(p, p_dt), conv(g, g_dt, ls), conv(m, m_dt), conv(v, v_dt), **kw)
         assert_same(got, want, dbg, pre, f"random case {case}: n={n} dtypes={(p_dt, g_dt, m_dt, v_dt)}")
+
+
+def test_random_centralized_pieces_match_the_oracle(handle):
+    """Centralization (adamw.py:179-184) through both kernels that carry it: random row lengths
+    (shorter and longer than a lane's vector, a unit, a wave's run), pieces that start and end in the middle of
+    rows, 16-bit layouts (whole units take the fast kernel's centralizing instance) and layouts with
+    an fp32 array (generic kernel).  The means are arbitrary numbers: the kernels only consume them."""
+    rng = np.random.default_rng(777)
+    for case in range(60):
+        row_len = int(rng.choice([rng.integers(1, 8), rng.integers(8, 40), rng.integers(100, 5000), 4096,
+                                  8192 + rng.integers(-9, 9), rng.integers(20_000, 40_000)]))
+        rows = int(max(1, min(rng.integers(1, 60), 300_000 // row_len)))
+        total = rows * row_len
+        start = int(rng.integers(0, max(1, total // 2))) // 8 * 8 if rng.random() < 0.7 else 0
+        count = int(rng.integers(1, total - start + 1)) if rng.random() < 0.5 else total - start
+        wide = rng.random() < 0.25
+        p_dt = int(rng.choice([oracle.DT_BF16, oracle.DT_F16]))
+        g_dt = int(rng.choice([oracle.DT_BF16, oracle.DT_F16])) if not wide else oracle.DT_F32
+        mv_dt = int(rng.choice([oracle.DT_BF16, oracle.DT_F16]))
+        cen = float(rng.choice([1.0, 0.5, 0.3]))
+        p, g, m, v = oracle.synth_inputs(total, int(rng.integers(0, 1 << 30)))
+        means = (rng.standard_normal(rows) * 1e-3).astype(np.float32)
+        tdt = {oracle.DT_BF16: torch.bfloat16, oracle.DT_F16: torch.float16}
+
+        def conv(a, dt):
+            f = oracle.bf16_to_f32(a)
+            if dt == oracle.DT_F32:
+                return (f * np.float32(1.0009765625)).astype(np.float32)
+            return f.astype(np.float16).view(np.uint16) if dt == oracle.DT_F16 else a
+
+        def up(a, dt):
+            return torch.from_numpy(a.copy()).cuda() if dt == oracle.DT_F32 else dev16(a, tdt[dt])
+
+        hp = dict(HP0, lr=float(10 ** rng.uniform(-4, -2)))
+        step, seed, tid = int(rng.choice([1, 7, 1000])), int(rng.integers(0, 1 << 62)), int(rng.integers(0, 1 << 20))
+        arrs = [conv(p, p_dt), conv(g, g_dt), conv(m, mv_dt), conv(v, mv_dt)]
+        P, G, M, V = (up(a, dt) for a, dt in zip(arrs, (p_dt, g_dt, mv_dt, mv_dt)))
+        sl = slice(start, start + count)
+        e = F.Entry(p=P[sl], g=G[sl], m=M[sl], v=V[sl], step=step, scalars_idx=0, tensor_id=tid,
+                    row_mean=torch.from_numpy(means).cuda(), row_len=row_len, elem_offset=start)
+        F.step_resident(handle, [e], [F.make_scalars(step=step, centralization=cen, **hp)], seed=seed, explicit_noise=False)
+        torch.cuda.synchronize()
+
+        g32 = arrs[1][sl].astype(np.float32) if g_dt == oracle.DT_F32 else (
+            oracle.bf16_to_f32(arrs[1][sl]) if g_dt == oracle.DT_BF16 else arrs[1][sl].view(np.float16).astype(np.float32))
+        row_of = (np.arange(start, start + count) // row_len)
+        g32 = (g32 - (means[row_of] * np.float32(cen)).astype(np.float32)).astype(np.float32)
+        po, mo, vo = arrs[0][sl].copy(), arrs[2][sl].copy(), arrs[3][sl].copy()
+        oracle.step_tensor(po, g32, mo, vo, oracle.scalars_from_hparams(step=step, **hp), p_dtype=p_dt,
+                           g_dtype=oracle.DT_F32, m_dtype=mv_dt, v_dtype=mv_dt, seed=seed, step=step, tensor_id=tid,
+                           elem_offset=start)
+        what = f"case {case}: rows={rows} row_len={row_len} start={start} count={count} dtypes={(p_dt, g_dt, mv_dt)}"
+        for name, t, a in zip("pmv", (P, M, V), (po, mo, vo)):
+            np.testing.assert_array_equal(bits16(t)[sl], a, err_msg=f"{what} {name}")
+        # nothing outside the piece was touched
+        for name, t, a in zip("pmv", (P, M, V), (arrs[0], arrs[2], arrs[3])):
+            np.testing.assert_array_equal(bits16(t)[:start], a[:start], err_msg=f"{what} {name} before the piece")
+            np.testing.assert_array_equal(bits16(t)[start + count:], a[start + count:], err_msg=f"{what} {name} behind it")
