@@ -127,6 +127,25 @@ def test_unpinned_gradients_go_up_through_bounce_buffers(handle, chunk_elems):
     assert after["bytes"] - before["bytes"] == expect_bytes
 
 
+def test_unpinned_uploads_can_be_left_to_the_runtime(monkeypatch):
+    """RT_STREAM_BOUNCE_THREADS=0 (read when a handle first streams): no bounce buffers, no host
+    threads; the runtime stages the copies from ordinary CPU memory itself.  Same results."""
+    monkeypatch.setenv("RT_STREAM_BOUNCE_THREADS", "0")
+    h = N.Handle(0)
+    try:
+        n = 50_000
+        p, g, m, v = oracle.synth_inputs(n, 520)
+        e = F.Entry(p=host16(p), g=host16(g, pin=False), m=host16(m), v=host16(v), step=4, scalars_idx=0, tensor_id=3)
+        F.step_streamed(h, [e], [F.make_scalars(step=4, **HP0)], seed=8, explicit_noise=False, chunk_elems=8192)
+        assert h.streamed_bounce_stats() == {"calls": 0, "bytes": 0}
+        oracle.step_tensor(p, g, m, v, oracle.scalars_from_hparams(step=4, **HP0), seed=8, step=4, tensor_id=3)
+        for name, t, a in zip("pmv", (e.p, e.m, e.v), (p, m, v)):
+            np.testing.assert_array_equal(bits16(t), a, err_msg=name)
+    finally:
+        torch.cuda.synchronize()
+        h.close()
+
+
 def test_streamed_and_resident_agree_bit_for_bit(handle):
     n = 300_000
     p, g, m, v = oracle.synth_inputs(n, 95)
