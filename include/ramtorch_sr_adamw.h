@@ -80,7 +80,8 @@ typedef struct rt_tensor_desc {
     float* dbg_p;          /* optional device fp32[numel]: values before rounding (tests) */
     float* dbg_m;
     float* dbg_v;
-    const float* row_mean; /* centralization != 0: device fp32[numel/row_len] row means of g */
+    const float* row_mean; /* centralization != 0: device fp32[numel/row_len] row means of g (of the unscaled,
+                              unclipped gradient: a clip coefficient is applied to the mean as to the gradient) */
     uint64_t numel;
     uint64_t elem_offset;  /* index of element 0 inside the logical tensor; multiple of 8 */
     uint64_t row_len;      /* elements per row (dim 0 slice) when row_mean != NULL */

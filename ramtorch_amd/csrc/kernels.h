@@ -341,6 +341,15 @@ __device__ __forceinline__ void scale_grads(float (&g)[8], const UpdateCtx& c) {
     }
 }
 
+// What centralization subtracts from every gradient element of a row (adamw.py:179-184:
+// grad.sub_(mean.mul_(c)), the product rounded before it is subtracted).  `mean` is the row mean of
+// the unscaled gradient; with a clip coefficient the gradient has been multiplied by it, and so is
+// its mean (clipping first and centralizing afterwards is what clip_grad_norm_ followed by step() does).
+__device__ __forceinline__ float cen_term(float mean, const rt_scalars& s, bool do_clip, float coef) {
+    if (do_clip) mean = mean * coef;
+    return mean * s.centralization;
+}
+
 // ---------------------------------------------------------------------------
 // Launch-uniform set-up shared by the update kernels.
 // ---------------------------------------------------------------------------
@@ -540,7 +549,7 @@ __global__ __launch_bounds__(kThreads) void sr_adamw_fast_kernel(const LaunchArg
         scale_grads(g, c);
         if constexpr (CEN) {
             // grad.sub_(mean.mul_(c)): the product is rounded, then subtracted
-            const float mc0 = cur.mean0 * c.s.centralization, mc1 = cur.mean1 * c.s.centralization;
+            const float mc0 = cen_term(cur.mean0, c.s, c.do_clip, c.coef), mc1 = cen_term(cur.mean1, c.s, c.do_clip, c.coef);
 #pragma unroll
             for (int j = 0; j < 8; ++j) g[j] = g[j] - (cur.rem + (uint32_t)j < row_len ? mc0 : mc1);
         }
@@ -770,7 +779,7 @@ __global__ __launch_bounds__(kThreads) void sr_adamw_generic_kernel(const Launch
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 if (i + j < n) {
-                    const float mc = ldg32f(t.row_mean + row * 4) * c.s.centralization;
+                    const float mc = cen_term(ldg32f(t.row_mean + row * 4), c.s, c.do_clip, c.coef);
                     g[j] = g[j] - mc;
                 }
                 if (++rem == t.row_len) {
@@ -945,7 +954,7 @@ __global__ __launch_bounds__(kThreads) void sr_adamw_any_kernel(const LaunchArgs
             if (do_unscale) g = g * s.inv_loss_scale;
             if (do_clip) g = g * coef;
             if (t.row_mean != 0) {
-                const float mc = ldg32f(t.row_mean + row * 4) * s.centralization;
+                const float mc = cen_term(ldg32f(t.row_mean + row * 4), s, do_clip, coef);
                 g = g - mc;
                 if (++rem == t.row_len) {
                     rem = 0;

@@ -550,8 +550,6 @@ class AdamW(Optimizer):
                 e = F.Entry(p=arrays[0], g=g, m=arrays[1], v=arrays[2], step=step, scalars_idx=si,
                             tensor_id=r.tensor_id)
                 if cen != 0:
-                    if self.max_grad_norm is not None:
-                        raise NotImplementedError("centralization together with max_grad_norm")
                     if not g.is_cuda:
                         g = g.to(f"cuda:{dev}", non_blocking=True)
                         e.g = g
