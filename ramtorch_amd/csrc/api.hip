@@ -1270,16 +1270,31 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
                 st.bounce[a][k] = nullptr;
             }
             st.bounce_cap[a] = 0;
-            for (int k = 0; k < kBounce; ++k) {
-                hipError_t e = hipHostMalloc(&st.bounce[a][k], want, hipHostMallocDefault);
-                if (e != hipSuccess) {
+            bool got_all = true;
+            for (int k = 0; k < kBounce && got_all; ++k) {
+                if (hipHostMalloc(&st.bounce[a][k], want, hipHostMallocDefault) != hipSuccess) {
+                    (void)hipGetLastError();
                     st.bounce[a][k] = nullptr;
-                    return fail(RT_ENOMEM, "hipHostMalloc(%zu) for a bounce buffer failed: %s", want, hipGetErrorString(e));
+                    got_all = false;
                 }
+            }
+            if (!got_all) {
+                // No pinned memory to be had (a locked-memory limit, say): this call leaves the unpinned
+                // copies to the runtime, which is slower but needs nothing from us.
+                for (int k = 0; k < kBounce; ++k) {
+                    if (st.bounce[a][k]) (void)hipHostFree(st.bounce[a][k]);
+                    st.bounce[a][k] = nullptr;
+                }
+                paced = false;
+                break;
             }
             st.bounce_cap[a] = want;
         }
-        ++st.paced_calls;
+        if (paced) {
+            ++st.paced_calls;
+        } else {
+            std::fill(unpinned.begin(), unpinned.end(), (uint8_t)0);
+        }
     }
 
     // ---- descriptors of every piece (pointers into staging for host-resident arrays), and the
