@@ -222,6 +222,15 @@ int rt_row_means(rt_handle* h, const void* g, int g_dtype, uint64_t rows, uint64
                  float inv_loss_scale, float* d_row_mean, void* stream);
 
 /*
+ * The same for many gradients in one launch: for every tensor with a non-NULL
+ * row_mean, row_mean[r] = mean of row r of g (numel / row_len rows of row_len
+ * elements, numel a multiple of row_len; row_mean is written, not read).  Only
+ * g, g_dtype, numel, row_len and row_mean of a descriptor are used.  Same
+ * summation, and so the same bits, as rt_row_means.
+ */
+int rt_row_means_multi(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, float inv_loss_scale, void* stream);
+
+/*
  * copy_stochastic_(target, source, seed) of adamw.py:6-30: fp32 device source
  * -> bf16 device target.  noise == NULL: Philox keyed by seed; else explicit
  * 16-bit noise per element.

@@ -30,7 +30,7 @@ EXPORTS = (
     "rt_stream_probe", "rt_streamed_timeline", "rt_streamed_plan",
     "rt_step_streamed_async", "rt_streamed_wait", "rt_streamed_completed",
     "rt_grad_norm_static", "rt_host_link_probe", "rt_selftest_sqrt", "rt_dev_hold", "rt_dev_release",
-    "rt_streamed_bounce_stats",
+    "rt_streamed_bounce_stats", "rt_row_means_multi",
 )
 
 
@@ -130,6 +130,8 @@ def lib() -> ctypes.CDLL:
     L.rt_dev_release.argtypes = [vp, vp]
     L.rt_selftest_sqrt.restype = i32
     L.rt_selftest_sqrt.argtypes = [vp, ctypes.POINTER(u64)]
+    L.rt_row_means_multi.restype = i32
+    L.rt_row_means_multi.argtypes = [vp, descs, u32, ctypes.c_float, vp]
     L.rt_row_means.restype = i32
     L.rt_row_means.argtypes = [vp, vp, i32, u64, u64, ctypes.c_float, vp, vp]
     L.rt_sr_copy.restype = i32
@@ -266,6 +268,10 @@ class Handle:
         with self._lock:
             check(lib().rt_selftest_sqrt(self.ptr, ctypes.byref(n)))
         return n.value
+
+    def row_means_multi(self, descs, n, inv_loss_scale, stream=0):
+        with self._lock:
+            check(lib().rt_row_means_multi(self.ptr, descs, n, inv_loss_scale, stream))
 
     def row_means(self, g, g_dtype, rows, row_len, inv_loss_scale, d_row_mean, stream=0):
         with self._lock:

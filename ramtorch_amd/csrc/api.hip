@@ -184,6 +184,7 @@ struct rt_handle {
     void* static_scratch = nullptr;       // this device's copy of `scratch`
     std::vector<NormEntry> norm_entries;  // host image of the table of rt_grad_norm_static
     std::vector<NormEntry> norm_table;    // the same for rt_grad_norm
+    std::vector<RowMeanEntry> rowmean_table;  // host image of the table of rt_row_means_multi
     // The table image of the most recent rt_step_multi call, kept so that a call over the same tensors
     // (same addresses, sizes, types; every step count advanced by one common amount) rebuilds only
     // the per-step scalars.
@@ -982,6 +983,49 @@ int rt_row_means(rt_handle* h, const void* g, int g_dtype, uint64_t rows, uint64
         default: return fail(RT_EINVAL, "g_dtype %d unknown", g_dtype);
     }
     HIP_TRY(hipGetLastError());
+    return RT_OK;
+}
+
+int rt_row_means_multi(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, float inv_loss_scale, void* stream_) {
+    if (!h) return fail(RT_EINVAL, "handle is NULL");
+    if (n > 0 && !descs) return fail(RT_EINVAL, "descs is NULL");
+    hipStream_t stream = (hipStream_t)stream_;
+    HIP_TRY(hipSetDevice(h->device));
+    std::vector<RowMeanEntry>& tab = h->rowmean_table;
+    tab.clear();
+    uint64_t rows_total = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        const rt_tensor_desc& d = descs[i];
+        if (d.numel == 0 || !d.row_mean) continue;
+        if (!d.g || d.row_len == 0 || d.numel % d.row_len != 0)
+            return fail(RT_EINVAL, "tensor %u: NULL gradient, or numel %llu is not a multiple of row_len %llu", i,
+                        (unsigned long long)d.numel, (unsigned long long)d.row_len);
+        if (d.g_dtype > RT_DT_F16) return fail(RT_EINVAL, "tensor %u: g_dtype %d (need bf16, f32 or f16)", i, d.g_dtype);
+        if (d.host_mask & RT_HOST_G) return fail(RT_EINVAL, "tensor %u: the gradient must be device resident", i);
+        if ((uintptr_t)d.g % dtype_size(d.g_dtype)) return fail(RT_EINVAL, "tensor %u: gradient pointer not aligned", i);
+        RowMeanEntry e;
+        e.g = (uint64_t)d.g;
+        e.out = (uint64_t)d.row_mean;
+        e.row_len = d.row_len;
+        e.first_row = (uint32_t)rows_total;
+        e.dtype = (uint32_t)d.g_dtype;
+        tab.push_back(e);
+        rows_total += d.numel / d.row_len;
+        if (rows_total > kMaxGrid) return fail(RT_EUNSUPPORTED, "more than %llu rows in one call", (unsigned long long)kMaxGrid);
+    }
+    if (rows_total == 0) return RT_OK;
+    // the table goes through a staging slot, like the tables of the update
+    Plan plan;
+    plan.bytes = tab.size() * sizeof(RowMeanEntry);
+    h->image.assign((const uint8_t*)tab.data(), (const uint8_t*)tab.data() + plan.bytes);
+    TableSlot* slot = nullptr;
+    int rc = stage_image(h, plan, h->image.data(), 0, stream, &slot);
+    if (rc != RT_OK) return rc;
+    hipLaunchKernelGGL(row_mean_table_kernel, dim3((uint32_t)rows_total), dim3(kThreads), 0, stream,
+                       (const RowMeanEntry*)slot->dev.ptr, (uint32_t)tab.size(), inv_loss_scale);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipEventRecord(slot->done, stream));
+    slot->in_flight = true;
     return RT_OK;
 }
 

@@ -1276,13 +1276,9 @@ __global__ __launch_bounds__(kThreads) void grad_norm_finish_kernel(const double
     }
 }
 
-// Row means for centralization: one workgroup per row.
+// Row means for centralization: one workgroup per row.  The sum of one row, in every thread:
 template <int GDT>
-__global__ __launch_bounds__(kThreads) void row_mean_kernel(uint64_t g, uint64_t row_len, float inv_loss_scale,
-                                                            float* __restrict__ out) {
-    __shared__ float lds[kThreads / 64];
-    const uint64_t row = blockIdx.x;
-    const uint64_t base = row * row_len;
+__device__ __forceinline__ float row_sum(uint64_t g, uint64_t base, uint64_t row_len, float inv_loss_scale, float* lds) {
     const bool aligned = (g & 15u) == 0 && (row_len % kVec) == 0;
     float acc = 0.0f;
     for (uint64_t c = (uint64_t)threadIdx.x * kVec; c < row_len; c += (uint64_t)kThreads * kVec) {
@@ -1293,8 +1289,45 @@ __global__ __launch_bounds__(kThreads) void row_mean_kernel(uint64_t g, uint64_t
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc = acc + x[j] * inv_loss_scale;
     }
-    const float sum = block_sum(acc, lds);
+    return block_sum(acc, lds);
+}
+
+template <int GDT>
+__global__ __launch_bounds__(kThreads) void row_mean_kernel(uint64_t g, uint64_t row_len, float inv_loss_scale,
+                                                            float* __restrict__ out) {
+    __shared__ float lds[kThreads / 64];
+    const uint64_t row = blockIdx.x;
+    const float sum = row_sum<GDT>(g, row * row_len, row_len, inv_loss_scale, lds);
     if (threadIdx.x == 0) out[row] = sum / (float)row_len;
+}
+
+// The same for many gradients in one launch: workgroup b takes row b of the rows of all gradients
+// counted through, and finds its gradient by binary search over the first-row numbers.
+struct alignas(16) RowMeanEntry {
+    uint64_t g;
+    uint64_t out;        // fp32[rows] of this gradient
+    uint64_t row_len;
+    uint32_t first_row;  // number of this gradient's first row in the launch
+    uint32_t dtype;
+};
+static_assert(sizeof(RowMeanEntry) == 32, "RowMeanEntry layout");
+
+__global__ __launch_bounds__(kThreads) void row_mean_table_kernel(const RowMeanEntry* __restrict__ table, uint32_t n,
+                                                                  float inv_loss_scale) {
+    __shared__ float lds[kThreads / 64];
+    const uint32_t row = blockIdx.x;
+    uint32_t lo = 0, hi = n;  // the entry with the largest first_row <= row
+    while (hi - lo > 1) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (table[mid].first_row <= row) lo = mid; else hi = mid;
+    }
+    const RowMeanEntry e = table[lo];
+    const uint64_t r = row - e.first_row;
+    float sum;
+    if (e.dtype == RT_DT_BF16) sum = row_sum<RT_DT_BF16>(e.g, r * e.row_len, e.row_len, inv_loss_scale, lds);
+    else if (e.dtype == RT_DT_F32) sum = row_sum<RT_DT_F32>(e.g, r * e.row_len, e.row_len, inv_loss_scale, lds);
+    else sum = row_sum<RT_DT_F16>(e.g, r * e.row_len, e.row_len, inv_loss_scale, lds);
+    if (threadIdx.x == 0) ((RT_GLOBAL float*)e.out)[r] = sum / (float)e.row_len;
 }
 
 }  // namespace rt

@@ -227,3 +227,30 @@ def row_means(handle: N.Handle, g: torch.Tensor, rows: int, row_len: int, inv_lo
     handle.row_means(g.data_ptr(), dtype_code(g.dtype, "grad"), rows, row_len, float(inv_loss_scale),
                      out.data_ptr(), stream)
     return out
+
+
+def row_means_multi(handle: N.Handle, jobs: Sequence[Tuple[Entry, int, int]], inv_loss_scale: float = 1.0,
+                    stream: Optional[int] = None) -> None:
+    """Row means of the GPU gradients of many entries in one launch.  ``jobs`` holds
+    (entry, rows, row_len); every entry gets ``row_mean`` (a view into one fp32 buffer) and ``row_len``."""
+    jobs = [j for j in jobs if j[1] > 0 and j[2] > 0]
+    if not jobs:
+        return
+    dev = jobs[0][0].g.device
+    buf = torch.empty(sum(rows for _, rows, _ in jobs), dtype=torch.float32, device=dev)
+    d = np.zeros(len(jobs), DESC_DTYPE)
+    off = 0
+    for k, (e, rows, row_len) in enumerate(jobs):
+        if not e.g.is_cuda or not e.g.is_contiguous():
+            raise ValueError("row_means_multi needs contiguous CUDA gradients")
+        e.row_mean = buf[off:off + rows]
+        e.row_len = row_len
+        off += rows
+        d["g"][k] = e.g.data_ptr()
+        d["g_dtype"][k] = dtype_code(e.g.dtype, "grad")
+        d["numel"][k] = rows * row_len
+        d["row_len"][k] = row_len
+        d["row_mean"][k] = e.row_mean.data_ptr()
+    if stream is None:
+        stream = torch.cuda.current_stream(handle.device).cuda_stream
+    handle.row_means_multi(_descs_ptr(d), len(jobs), float(inv_loss_scale), stream)

@@ -456,6 +456,7 @@ class AdamW(Optimizer):
                 and sum(len(g["params"]) for g in self.param_groups) >= self.gather_min_tensors):
             gather = G.module()
         gathered: Dict[int, list] = {}    # dev -> [descriptor buffer, rows used]
+        cen_jobs: Dict[int, list] = {}    # dev -> [(entry, rows, row_len)] of gradients to centralize
 
         for gi, group in enumerate(self.param_groups):
             beta1, beta2 = group["betas"]
@@ -553,13 +554,23 @@ class AdamW(Optimizer):
                     if not g.is_cuda:
                         g = g.to(f"cuda:{dev}", non_blocking=True)
                         e.g = g
-                    e.row_mean, e.row_len = self._row_means(g, dev, inv_loss_scale)
+                    if getattr(self, "noise_source", "philox") == "reference" and inv_loss_scale == 1.0:
+                        e.row_mean, e.row_len = self._row_means(g, dev, inv_loss_scale)   # torch's own mean
+                    elif g.numel():
+                        # adamw.py:179-184: mean over every dim but the first (over all of them for 0-d / 1-d);
+                        # the rows of all such gradients of the step are summed in one launch below
+                        rows = g.shape[0] if g.dim() >= 2 else 1
+                        cen_jobs.setdefault(dev, []).append((e, rows, g.numel() // rows if rows else 0))
                 if noise is not None and p in noise:
                     e.noise = tuple(noise[p])
                 if debug_out is not None and p in debug_out:
                     e.dbg = tuple(debug_out[p])
                 on_gpu = e.p.is_cuda and e.g.is_cuda and e.m.is_cuda and e.v.is_cuda
                 (resident if on_gpu else streamed).setdefault(dev, []).append(e)
+
+        for dev, jobs in cen_jobs.items():
+            with torch.cuda.device(dev):
+                F.row_means_multi(_handle(dev), jobs, inv_loss_scale)   # writes fresh buffers only
 
         # ---- everything that can still raise for a bad argument happens before the first launch
         explicit = noise is not None

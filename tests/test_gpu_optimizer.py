@@ -373,6 +373,31 @@ def test_centralization_in_pieces_equals_whole(shape):
         np.testing.assert_array_equal(a, b)
 
 
+def test_row_means_of_many_gradients_in_one_launch():
+    """rt_row_means_multi = rt_row_means tensor by tensor, bit for bit (same summation), for row
+    lengths around the vector width, unaligned views and every gradient dtype."""
+    rng = np.random.default_rng(11)
+    h = N.Handle(0)
+    jobs, singles = [], []
+    for k in range(40):
+        row_len = int(rng.choice([1, 3, 8, 12, 100, 511, 4096, 5000]))
+        rows = int(rng.integers(1, 40))
+        dt = [torch.bfloat16, torch.float32, torch.float16][k % 3]
+        off = int(rng.integers(0, 3))                     # a view that does not start on 16 bytes
+        g = (torch.randn(rows * row_len + off, device="cuda") * 1e-3).to(dt)[off:]
+        e = F.Entry(p=g, g=g, m=g, v=g, step=1, scalars_idx=0, tensor_id=k)
+        jobs.append((e, rows, row_len))
+        singles.append(F.row_means(h, g, rows, row_len, 0.5))
+    F.row_means_multi(h, jobs, 0.5)
+    torch.cuda.synchronize()
+    for k, ((e, rows, row_len), one) in enumerate(zip(jobs, singles)):
+        assert e.row_len == row_len and e.row_mean.numel() == rows
+        assert nmis(e.row_mean, one) == 0, (k, rows, row_len)
+        want = (e.g.double().view(rows, row_len) * 0.5).mean(dim=1).cpu().numpy()
+        np.testing.assert_allclose(e.row_mean.cpu().numpy(), want, rtol=3e-6, atol=1e-9)
+    h.close()
+
+
 def test_clip_with_centralization():
     """max_grad_norm and centralization together (neither the combination nor the clip is in the
     reference): the clip coefficient scales the gradient and its row means alike, as clip_grad_norm_
