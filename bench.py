@@ -540,6 +540,10 @@ def main() -> int:
             r["steps"] = k
             sec[w] = r
 
+    for w, r in sec.items():
+        if w in RESIDENT and r["roofline"].get("achieved") and main_res["roofline"].get("achieved"):
+            r["roofline"]["rate_vs_main_workload"] = r["roofline"]["achieved"] / main_res["roofline"]["achieved"]
+
     out = {
         "metric": METRIC, "value": main_res["elements_per_s"], "unit": "elements/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"], "higher_is_better": True,
