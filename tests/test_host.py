@@ -423,3 +423,44 @@ def test_bench_refuses_more_than_one_gpu():
                          capture_output=True, text=True, timeout=120)
     assert res.returncode != 0
     assert "ONE GPU" in res.stderr and res.stdout.strip() == ""
+
+
+def test_copy_pool_copies_every_byte_and_waits_per_group(tmp_path):
+    """The host threads that fill the streamed path's bounce buffers (csrc/copy_pool.h): many groups
+    of copies of odd sizes submitted at once, each waited for on its own, compared byte for byte;
+    waiting on a group with nothing in it returns; the pool shuts down with idle workers."""
+    src = tmp_path / "pool.cpp"
+    src.write_text(r'''
+#include "copy_pool.h"
+#include <cstdio>
+#include <random>
+int main() {
+    std::mt19937_64 rng(7);
+    const size_t sizes[] = {0, 1, 63, 4096, (2u << 20) - 1, (2u << 20), (2u << 20) + 1, 9u << 20};
+    std::vector<std::vector<uint8_t>> from, to;
+    for (int rep = 0; rep < 3; ++rep)
+        for (size_t n : sizes) {
+            from.emplace_back(n);
+            to.emplace_back(n, (uint8_t)0);
+            for (auto& b : from.back()) b = (uint8_t)rng();
+        }
+    {
+        rt::CopyPool pool(5);
+        std::vector<rt::CopyPool::Group> groups(from.size());
+        rt::CopyPool::Group empty;
+        pool.wait(&empty);
+        for (size_t i = 0; i < from.size(); ++i) pool.submit(&groups[i], to[i].data(), from[i].data(), from[i].size());
+        for (size_t i = from.size(); i-- > 0;) {  // waited for in the opposite order
+            pool.wait(&groups[i]);
+            if (to[i] != from[i]) { std::printf("group %zu differs\n", i); return 1; }
+        }
+    }
+    { rt::CopyPool idle(3); }
+    std::printf("ok\n");
+    return 0;
+}
+''')
+    exe = tmp_path / "pool"
+    subprocess.check_call(["g++", "-std=c++17", "-O1", "-Wall", "-Werror", "-pthread", "-fsanitize=thread",
+                           "-I", os.path.join(ROOT, "ramtorch_amd", "csrc"), str(src), "-o", str(exe)])
+    assert subprocess.check_output([str(exe)], text=True).strip() == "ok"
