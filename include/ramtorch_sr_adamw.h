@@ -43,6 +43,9 @@ extern "C" {
 #define RT_HOST_G 2u
 #define RT_HOST_M 4u
 #define RT_HOST_V 8u
+/* Host arrays of this tensor may still be written by work queued on the caller's stream: uploads wait for
+ * that work.  Implied for a gradient in pinned host memory; see rt_step_streamed. */
+#define RT_HOST_ORDERED 16u
 
 /*
  * Per-(param group, step) constants: the Python doubles of
@@ -140,6 +143,12 @@ int rt_step_multi(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const r
  * Results are bit-identical to rt_step_multi on the same data.
  * d_clip_coef / d_skip: as for rt_step_multi (device pointers, may be NULL);
  * they must be final for work queued on `stream` before the call.
+ * Ordering against `stream`: the update kernels always wait for the work queued
+ * on it.  The uploads wait for it only for tensors whose gradient lies in pinned
+ * host memory (an asynchronous device-to-host copy on `stream` may still be
+ * filling it, as after grad.to("cpu", non_blocking=True)) or that carry
+ * RT_HOST_ORDERED; host-resident p / m / v are otherwise taken to be final in
+ * host memory when the call is made (they are the optimizer's own to write).
  * Host arrays need not be pinned: the gradients that ramtorch's Linear.backward
  * leaves in ordinary CPU memory (linear.py:416-427, shipped up at adamw.py:167)
  * are copied into pinned bounce buffers of the handle (4 per array, one chunk

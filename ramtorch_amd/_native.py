@@ -22,6 +22,7 @@ RT_EINVAL, RT_EHIP, RT_ENOMEM, RT_EUNSUPPORTED = -1, -2, -3, -4
 RT_DT_BF16, RT_DT_F32, RT_DT_F16, RT_DT_F64 = 0, 1, 2, 3
 RT_NOISE_PHILOX, RT_NOISE_EXPLICIT = 0, 1
 RT_HOST_P, RT_HOST_G, RT_HOST_M, RT_HOST_V = 1, 2, 4, 8
+RT_HOST_ORDERED = 16
 
 #: every symbol the header declares
 EXPORTS = (

@@ -1285,17 +1285,20 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
     //      the pipeline one chunk at a time (at most kPacedInFlight on the streams, see below)
     //      instead of queuing everything up front.  Left to the runtime, such a copy is staged
     //      inside hipMemcpyAsync while the calling thread waits, and nothing else gets queued.
-    std::vector<uint8_t> unpinned(n, 0);  // bit a: array a of the tensor is host memory that is not pinned
+    std::vector<uint8_t> unpinned_probe(n, 0);  // bit a: array a of the tensor is host memory that is not pinned
+    for (uint32_t i = 0; i < n; ++i) {
+        const rt_tensor_desc& d = descs[i];
+        if (d.numel == 0) continue;
+        const void* host[4] = {d.p, d.g, d.m, d.v};
+        for (int a = 0; a < 4; ++a)
+            if ((d.host_mask & (1u << a)) && !is_pinned_host(host[a])) unpinned_probe[i] |= (uint8_t)(1u << a);
+    }
+    std::vector<uint8_t> unpinned(n, 0);  // the same, for the arrays that go up through bounce buffers
     bool paced = false;
-    if (st.bounce_threads > 0)
-        for (uint32_t i = 0; i < n; ++i) {
-            const rt_tensor_desc& d = descs[i];
-            if (d.numel == 0) continue;
-            const void* host[4] = {d.p, d.g, d.m, d.v};
-            for (int a = 0; a < 4; ++a)
-                if ((d.host_mask & (1u << a)) && !is_pinned_host(host[a])) unpinned[i] |= (uint8_t)(1u << a);
-            paced |= unpinned[i] != 0;
-        }
+    if (st.bounce_threads > 0) {
+        unpinned = unpinned_probe;
+        for (uint32_t i = 0; i < n; ++i) paced |= unpinned[i] != 0;
+    }
     if (paced) {
         // the bounce buffers and the chunk counter are shared with earlier calls: let those finish
         if (st.pending) {
@@ -1412,8 +1415,23 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
     memcpy(tab.host, blob.data(), blob.size());
 
     // grads (and anything else already queued by the caller) must be ready
+    // The kernels read device arrays (gradients above all) that work on the caller's stream may still
+    // be producing, so the compute stream always waits for it.  The upload stream waits only when it
+    // has to: a copy engine waiting on a compute stream's event was measured to stall the pipeline
+    // for 50 ms every few dozen chunks when updates are handed over chunk by chunk.  It has to when a
+    // gradient lies in pinned host memory, which an asynchronous copy on the caller's stream may still
+    // be filling (grad.to("cpu", non_blocking=True)), or when the caller asks for it (RT_HOST_ORDERED).
+    // Host memory that is not pinned cannot be the target of an asynchronous copy, and host-resident
+    // p / m / v are the optimizer's own to write.
+    bool upload_waits = false;
+    for (uint32_t i = 0; i < n && !upload_waits; ++i) {
+        const rt_tensor_desc& d = descs[i];
+        if (d.numel == 0) continue;
+        upload_waits = (d.host_mask & RT_HOST_ORDERED) != 0 ||
+                       ((d.host_mask & RT_HOST_G) != 0 && !(unpinned_probe[i] & RT_HOST_G));
+    }
     HIP_TRY(hipEventRecord(st.start, user));
-    HIP_TRY(hipStreamWaitEvent(st.h2d, st.start, 0));
+    if (upload_waits) HIP_TRY(hipStreamWaitEvent(st.h2d, st.start, 0));
     HIP_TRY(hipStreamWaitEvent(st.comp, st.start, 0));
     if (!blob.empty()) {
         const uint64_t n_vec = (blob.size() + 15) / 16;  // buffers are padded well past the blob

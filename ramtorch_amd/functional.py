@@ -76,6 +76,7 @@ class Entry:
     row_mean: Optional[torch.Tensor] = None
     row_len: int = 0
     elem_offset: int = 0
+    ordered: bool = False  # host arrays may still be written by work queued on the stream: uploads wait for it
     keep: list = field(default_factory=list)  # temporaries that must outlive the launch
 
 
@@ -131,6 +132,8 @@ def pack_descs(entries: Sequence[Entry], streamed: bool) -> np.ndarray:
                 mask |= bit
         if mask and not streamed:
             raise ValueError(f"tensor {i}: a CPU tensor reached the resident entry point")
+        if mask and e.ordered:
+            mask |= N.RT_HOST_ORDERED
         d["host_mask"][i] = mask
     return d
 

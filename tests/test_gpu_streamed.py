@@ -146,6 +146,33 @@ def test_unpinned_uploads_can_be_left_to_the_runtime(monkeypatch):
         h.close()
 
 
+@pytest.mark.parametrize("which", ["pinned gradient", "ordered parameter"])
+def test_uploads_wait_for_host_arrays_the_stream_is_still_filling(handle, which):
+    """A gradient in pinned host memory may still be on its way there (grad.to("cpu", non_blocking=True)
+    on a busy stream): the upload must wait for the caller's stream.  The same for a host parameter
+    when the caller says so (RT_HOST_ORDERED); without either, uploads do not wait."""
+    n = 3_000_000
+    p, g, m, v = oracle.synth_inputs(n, 530)
+    stale = torch.zeros(n, dtype=torch.bfloat16).pin_memory()
+    # everything is prepared first: a blocking copy further down would drain the stream
+    if which == "pinned gradient":
+        fresh = dev16(g)
+        e = F.Entry(p=host16(p), g=stale, m=host16(m), v=host16(v), step=6, scalars_idx=0, tensor_id=1)
+    else:
+        fresh = dev16(p)
+        e = F.Entry(p=stale, g=dev16(g), m=host16(m), v=host16(v), step=6, scalars_idx=0, tensor_id=1, ordered=True)
+    sc = [F.make_scalars(step=6, **HP0)]
+    busy = torch.randn(4096, 4096, device="cuda")
+    torch.cuda.synchronize()
+    for _ in range(150):                      # a hundred milliseconds of work ahead of the copy
+        busy = (busy @ busy) * 1e-4
+    stale.copy_(fresh, non_blocking=True)     # not there yet when the call below is made
+    F.step_streamed(handle, [e], sc, seed=12, explicit_noise=False, chunk_elems=1 << 20)
+    oracle.step_tensor(p, g, m, v, oracle.scalars_from_hparams(step=6, **HP0), seed=12, step=6, tensor_id=1)
+    for name, t, a in zip("pmv", (e.p, e.m, e.v), (p, m, v)):
+        np.testing.assert_array_equal(bits16(t), a, err_msg=name)
+
+
 def test_streamed_and_resident_agree_bit_for_bit(handle):
     n = 300_000
     p, g, m, v = oracle.synth_inputs(n, 95)
