@@ -207,6 +207,8 @@ def test_pack_descs_rejects_bad_inputs():
         F.pack_descs([e], streamed=False)
     d = F.pack_descs([e], streamed=True)
     assert d["host_mask"][0] == 15 and d["numel"][0] == 8 and d["p"][0] == e.p.data_ptr()
+    e.ordered = True   # host arrays the caller's stream may still be filling: uploads must wait for it
+    assert F.pack_descs([e], streamed=True)["host_mask"][0] == 15 | N.RT_HOST_ORDERED == 31
     with pytest.raises(ValueError, match="element counts"):
         F.pack_descs([F.Entry(p=t(8), g=t(9), m=t(8), v=t(8), step=1, scalars_idx=0, tensor_id=0)], streamed=True)
     # fp16 / fp64 params and states are valid (plain copy_ on write-back, adamw.py:208-222) ...
