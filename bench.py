@@ -39,9 +39,12 @@ ema~N(0,1e-4), ema_squared=N(0,1e-3)^2, stored bf16):
             post-accumulate hook
   offload_ref  the same set as the reference's own offload flow leaves it
             (linear.py:416-427 -> adamw.py:167): pinned CPU params and states
-            and the gradients on the CPU too (in ordinary, not pinned, memory, as
-            ``.to("cpu", non_blocking=True)`` allocates them); 8 bytes per element
-            go up the host link, 6 come down
+            and the gradients on the CPU too (in the pinned memory that
+            ``.to("cpu", non_blocking=True)`` allocates); 8 bytes per element
+            go up the host link, 6 come down.  Without the two embedding tensors
+            (6 979 584 000 elements): a process can pin about 64 GiB on the box.
+            Also timed with the gradients in ordinary CPU memory
+            (``unpinned_gradients``)
 """
 from __future__ import annotations
 
@@ -409,29 +412,61 @@ def run_host(workloads, args, steps, warmup):
     gmap = dict(zip(params, grads))
     results = {}
     link = None
+    if "offload_ref" in workloads:   # it rebuilds the optimizer on a subset: last
+        workloads = [w for w in workloads if w != "offload_ref"] + ["offload_ref"]
     for wl in workloads:
         cpu_grads = None
+        wl_shapes, wl_total = shapes, total
         if wl == "hooked":
             def one_step():
                 for p, g in zip(reversed(params), reversed(grads)):
                     opt.step_param(p, g)
                 opt.step()
         elif wl == "offload_ref":
-            # gradients where Linear.backward leaves them: ordinary CPU memory
-            cpu_grads = {p: g.to("cpu") for p, g in gmap.items()}
+            # Gradients where Linear.backward leaves them (linear.py:416-427): on the CPU, in the pinned memory
+            # that .to("cpu", non_blocking=True) allocates.  A process can pin about 64 GiB on the GPU box and
+            # torch's pinned allocator rounds every tensor up to a power of two, so 16 GB of pinned gradients do
+            # not fit next to the 48.2 GB of parameters and states: this workload runs without the two
+            # 525 M-element embedding tensors (whose 1.05 GB arrays cost 2 GiB of pinned memory each).  The new
+            # optimizer's states reuse the pinned blocks of the old one; what the embeddings held is unpinned.
+            keep = [i for i, s_ in enumerate(shapes) if numel(s_) < (1 << 28)]
+            wl_shapes = [shapes[i] for i in keep]
+            wl_params = [params[i] for i in keep]
+            wl_grads = [grads[i] for i in keep]
+            del opt, gmap
+            params = grads = None
+            gc.collect()
+            opt = ramtorch_amd.AdamW(wl_params, dtype=torch.bfloat16, **HP, storage_device="cpu", seed=1234,
+                                     stream_chunk_bytes=args.stream_chunk_mb << 20)
+            set_states(opt, wl_params, 100, warmup + 1, dev)
+            gc.collect()
+            torch._C._host_emptyCache()
+            wl_total = sum(numel(s_) for s_ in wl_shapes)
+            cpu_grads = {p: g.to("cpu", non_blocking=True) for p, g in zip(wl_params, wl_grads)}
+            torch.cuda.synchronize()
+            assert all(g.is_pinned() for g in cpu_grads.values())
             one_step = lambda: opt.step(grads=cpu_grads)
         else:
             one_step = lambda: opt.step(grads=gmap)
-        bounce0 = handle.streamed_bounce_stats()
         ms_per_step, _ = timed_steps(one_step, steps, warmup, handle, False)
-        bounce1 = handle.streamed_bounce_stats()
-        up = {"streamed": 6.0, "hooked": 6.0, "offload_ref": 8.0}[wl] * total
-        down = 6.0 * total
+        up = {"streamed": 6.0, "hooked": 6.0, "offload_ref": 8.0}[wl] * wl_total
+        down = 6.0 * wl_total
         secs = ms_per_step * 1e-3
         info = {"h2d_GBps": up / secs / 1e9, "d2h_GBps": down / secs / 1e9, "host_bytes_up": up, "host_bytes_down": down}
-        if bounce1["calls"] != bounce0["calls"]:
-            # host arrays that are not pinned went up through the library's pinned bounce buffers
-            info["bounced_bytes_per_step"] = (bounce1["bytes"] - bounce0["bytes"]) / (steps + warmup)
+        if wl == "offload_ref":
+            # the same with the gradients in ordinary (not pinned) CPU memory, as a plain .to("cpu") leaves
+            # them: they go up through the library's pinned bounce buffers, filled by host threads
+            del cpu_grads
+            gc.collect()
+            torch._C._host_emptyCache()
+            plain_grads = {p: g.to("cpu") for p, g in zip(wl_params, wl_grads)}
+            b0 = handle.streamed_bounce_stats()
+            ms2, _ = timed_steps(lambda: opt.step(grads=plain_grads), 2, 1, handle, False)
+            b1 = handle.streamed_bounce_stats()
+            info["unpinned_gradients"] = {"ms_per_step": ms2, "h2d_GBps": up / (ms2 * 1e-3) / 1e9,
+                                          "bounced_bytes_per_step": (b1["bytes"] - b0["bytes"]) / 3}
+            del plain_grads
+            cpu_grads = None
         if link is None:
             # same-run pinned-copy peaks with the same chunk size, each direction alone and both at
             # once (what the pipeline does in steady state), on the library's own copy streams
@@ -455,15 +490,16 @@ def run_host(workloads, args, steps, warmup):
                 info["d2h_chunk_ms"] = {"median": sorted(d2h)[len(d2h) // 2], "max": max(d2h), "last": d2h[-1]}
                 info["pipeline_ms"] = tl[-1][3] - tl[0][0]
         del cpu_grads
-        results[wl] = {"ms_per_step": ms_per_step, "elements_per_s": total / secs,
-                       "config": config_of(wl, shapes, total, 100, False), "host_link": info,
+        results[wl] = {"ms_per_step": ms_per_step, "elements_per_s": wl_total / secs,
+                       "config": config_of(wl, wl_shapes, wl_total, 100, False), "host_link": info,
                        "roofline": {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                                     "frac": None, "traffic": None, "note": "host-link bound; see host_link"}}
     for r in results.values():
         r["setup_seconds"] = setup_s
-    del opt, params, grads, gmap
+    del opt, params, grads
     gc.collect()
     torch.cuda.empty_cache()
+    torch._C._host_emptyCache()
     return results
 
 

@@ -1230,7 +1230,7 @@ struct FillGuard {
 static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
                             uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems,
                             const float* d_clip_coef, const uint32_t* d_skip, void* stream_, bool trace,
-                            uint64_t* ticket_out) {
+                            bool blocking, uint64_t* ticket_out) {
     if (!h) return fail(RT_EINVAL, "handle is NULL");
     int rc = validate(descs, n, scalars, n_scalars, noise_mode, /*allow_host=*/true);
     if (rc != RT_OK) return rc;
@@ -1431,7 +1431,13 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
                        ((d.host_mask & RT_HOST_G) != 0 && !(unpinned_probe[i] & RT_HOST_G));
     }
     HIP_TRY(hipEventRecord(st.start, user));
-    if (upload_waits) HIP_TRY(hipStreamWaitEvent(st.h2d, st.start, 0));
+    if (upload_waits) {
+        // A call that returns only when everything is done, with nothing of the pipeline running
+        // yet, may as well wait on the host: even one such wait on the upload stream per call was
+        // measured to cost most calls the same 50 ms.
+        if (blocking && !st.pending) HIP_TRY(hipStreamSynchronize(user));
+        else HIP_TRY(hipStreamWaitEvent(st.h2d, st.start, 0));
+    }
     HIP_TRY(hipStreamWaitEvent(st.comp, st.start, 0));
     if (!blob.empty()) {
         const uint64_t n_vec = (blob.size() + 15) / 16;  // buffers are padded well past the blob
@@ -1580,9 +1586,9 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
 static int streamed_enqueue(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
                             uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems,
                             const float* d_clip_coef, const uint32_t* d_skip, void* stream_, bool trace,
-                            uint64_t* ticket_out) {
+                            bool blocking, uint64_t* ticket_out) {
     const int rc = streamed_enqueue_impl(h, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, d_clip_coef,
-                                         d_skip, stream_, trace, ticket_out);
+                                         d_skip, stream_, trace, blocking, ticket_out);
     if (rc != RT_OK && h && h->st.ready) {
         char saved[sizeof(g_err)];
         memcpy(saved, g_err, sizeof(saved));
@@ -1605,7 +1611,7 @@ int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, cons
     const auto wall0 = std::chrono::steady_clock::now();
     const bool trace = h->timing;
     int rc = streamed_enqueue(h, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, d_clip_coef, d_skip,
-                              stream, trace, nullptr);
+                              stream, trace, /*blocking=*/true, nullptr);
     if (rc != RT_OK) return rc;
     // Host memory is final on return; device-resident arrays are final for the caller's stream.
     rc = streamed_wait(h);
@@ -1623,7 +1629,7 @@ int rt_step_streamed_async(rt_handle* h, const rt_tensor_desc* descs, uint32_t n
                            const float* d_clip_coef, const uint32_t* d_skip, void* stream, uint64_t* ticket) {
     if (!h) return fail(RT_EINVAL, "handle is NULL");
     return streamed_enqueue(h, descs, n, scalars, n_scalars, seed, noise_mode, chunk_elems, d_clip_coef, d_skip,
-                            stream, false, ticket);
+                            stream, false, /*blocking=*/false, ticket);
 }
 
 int rt_streamed_wait(rt_handle* h) {

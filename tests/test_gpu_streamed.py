@@ -146,8 +146,9 @@ def test_unpinned_uploads_can_be_left_to_the_runtime(monkeypatch):
         h.close()
 
 
+@pytest.mark.parametrize("blocking", [True, False])
 @pytest.mark.parametrize("which", ["pinned gradient", "ordered parameter"])
-def test_uploads_wait_for_host_arrays_the_stream_is_still_filling(handle, which):
+def test_uploads_wait_for_host_arrays_the_stream_is_still_filling(handle, which, blocking):
     """A gradient in pinned host memory may still be on its way there (grad.to("cpu", non_blocking=True)
     on a busy stream): the upload must wait for the caller's stream.  The same for a host parameter
     when the caller says so (RT_HOST_ORDERED); without either, uploads do not wait."""
@@ -167,7 +168,10 @@ def test_uploads_wait_for_host_arrays_the_stream_is_still_filling(handle, which)
     for _ in range(150):                      # a hundred milliseconds of work ahead of the copy
         busy = (busy @ busy) * 1e-4
     stale.copy_(fresh, non_blocking=True)     # not there yet when the call below is made
-    F.step_streamed(handle, [e], sc, seed=12, explicit_noise=False, chunk_elems=1 << 20)
+    # the call that returns when all is done waits for the stream on the host, the asynchronous one on the GPU
+    F.step_streamed(handle, [e], sc, seed=12, explicit_noise=False, chunk_elems=1 << 20, wait=blocking)
+    if not blocking:
+        handle.streamed_wait()
     oracle.step_tensor(p, g, m, v, oracle.scalars_from_hparams(step=6, **HP0), seed=12, step=6, tensor_id=1)
     for name, t, a in zip("pmv", (e.p, e.m, e.v), (p, m, v)):
         np.testing.assert_array_equal(bits16(t), a, err_msg=name)
