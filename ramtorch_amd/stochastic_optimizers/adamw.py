@@ -120,7 +120,8 @@ class AdamW(Optimizer):
             ``ramtorch_amd/placement.py``; the outcome is in ``state_placement_report``).
             While it searches, the constructor occupies up to half of the free device memory
             (at most 112 GiB, for at most 8 s) through the library and gives all of it back;
-            torch's caching allocator only ever sees the two pools.
+            torch's caching allocator only ever sees the first pool (the second is memory held
+            through the library, wrapped as a tensor, and released with its last view).
             "plain" allocates every state tensor on its own, as the reference does.
     """
 
