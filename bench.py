@@ -234,6 +234,14 @@ def set_states(opt, params, first_step, warmup, dev):
         st["ema_squared"].copy_(fill_tensor(p.shape, "v", 1234 + 4 * i + 3, st["ema_squared"].dtype, dev))
 
 
+def _unpin_free_host_blocks():
+    """Give the pinned host blocks that torch's allocator holds but nothing uses back to the system."""
+    import torch
+    fn = getattr(torch._C, "_host_emptyCache", None)
+    if fn is not None:
+        fn()
+
+
 def timed_steps(one_step, steps, warmup, handle, resident):
     import torch
     for _ in range(warmup):
@@ -440,7 +448,7 @@ def run_host(workloads, args, steps, warmup):
                                      stream_chunk_bytes=args.stream_chunk_mb << 20)
             set_states(opt, wl_params, 100, warmup + 1, dev)
             gc.collect()
-            torch._C._host_emptyCache()
+            _unpin_free_host_blocks()
             wl_total = sum(numel(s_) for s_ in wl_shapes)
             cpu_grads = {p: g.to("cpu", non_blocking=True) for p, g in zip(wl_params, wl_grads)}
             torch.cuda.synchronize()
@@ -458,7 +466,7 @@ def run_host(workloads, args, steps, warmup):
             # them: they go up through the library's pinned bounce buffers, filled by host threads
             del cpu_grads
             gc.collect()
-            torch._C._host_emptyCache()
+            _unpin_free_host_blocks()
             plain_grads = {p: g.to("cpu") for p, g in zip(wl_params, wl_grads)}
             b0 = handle.streamed_bounce_stats()
             ms2, _ = timed_steps(lambda: opt.step(grads=plain_grads), 2, 1, handle, False)
@@ -499,7 +507,7 @@ def run_host(workloads, args, steps, warmup):
     del opt, params, grads
     gc.collect()
     torch.cuda.empty_cache()
-    torch._C._host_emptyCache()
+    _unpin_free_host_blocks()
     return results
 
 
