@@ -450,9 +450,18 @@ def run_host(workloads, args, steps, warmup):
             gc.collect()
             _unpin_free_host_blocks()
             wl_total = sum(numel(s_) for s_ in wl_shapes)
-            cpu_grads = {p: g.to("cpu", non_blocking=True) for p, g in zip(wl_params, wl_grads)}
-            torch.cuda.synchronize()
-            assert all(g.is_pinned() for g in cpu_grads.values())
+            pinned_ok = True
+            try:
+                cpu_grads = {p: g.to("cpu", non_blocking=True) for p, g in zip(wl_params, wl_grads)}
+                torch.cuda.synchronize()
+                pinned_ok = all(g.is_pinned() for g in cpu_grads.values())
+            except RuntimeError:   # no more memory to pin on this machine
+                pinned_ok = False
+            if not pinned_ok:      # measured with ordinary CPU memory only, and said so
+                cpu_grads = None
+                gc.collect()
+                _unpin_free_host_blocks()
+                cpu_grads = {p: g.to("cpu") for p, g in zip(wl_params, wl_grads)}
             one_step = lambda: opt.step(grads=cpu_grads)
         else:
             one_step = lambda: opt.step(grads=gmap)
@@ -462,6 +471,8 @@ def run_host(workloads, args, steps, warmup):
         secs = ms_per_step * 1e-3
         info = {"h2d_GBps": up / secs / 1e9, "d2h_GBps": down / secs / 1e9, "host_bytes_up": up, "host_bytes_down": down}
         if wl == "offload_ref":
+            info["gradients_pinned"] = pinned_ok
+        if wl == "offload_ref" and pinned_ok:
             # the same with the gradients in ordinary (not pinned) CPU memory, as a plain .to("cpu") leaves
             # them: they go up through the library's pinned bounce buffers, filled by host threads
             del cpu_grads
