@@ -53,7 +53,8 @@ struct ChunkRef {
 // the same position.  A few hundred bytes for a transformer's parameter set, so the search runs
 // out of cache, where a per-workgroup table entry would be a fresh HBM line.
 // (Units of two or four chunks per workgroup were measured 1.5 % and 2.5 % slower on the 8B set.)
-constexpr uint32_t kFastUnitElems = kChunkElems;
+constexpr int kFastIters = kItersPerChunk;           // vectors per lane per fast unit
+constexpr uint32_t kFastUnitElems = kThreads * kVec * kFastIters;
 
 // Piece kernel: a wavefront owns one piece of at most kPieceElems consecutive elements -- a whole
 // short tensor, or part of what a long tensor leaves over after its whole fast units.  The record
