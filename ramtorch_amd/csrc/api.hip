@@ -966,22 +966,17 @@ int rt_row_means(rt_handle* h, const void* g, int g_dtype, uint64_t rows, uint64
     if (rows == 0) return RT_OK;
     if (!g || !d_row_mean || row_len == 0) return fail(RT_EINVAL, "NULL pointer or empty row");
     if (rows > 0x7FFFFFFFull) return fail(RT_EUNSUPPORTED, "too many rows");
+    if (g_dtype < 0 || g_dtype > RT_DT_F16) return fail(RT_EINVAL, "g_dtype %d unknown", g_dtype);
+    if ((uintptr_t)g % dtype_size(g_dtype)) return fail(RT_EINVAL, "gradient pointer not aligned to its element size");
     hipStream_t stream = (hipStream_t)stream_;
     HIP_TRY(hipSetDevice(h->device));
-    switch (g_dtype) {
-        case RT_DT_BF16:
-            hipLaunchKernelGGL(row_mean_kernel<RT_DT_BF16>, dim3((uint32_t)rows), dim3(kThreads), 0, stream,
-                               (uint64_t)g, row_len, inv_loss_scale, d_row_mean);
-            break;
-        case RT_DT_F32:
-            hipLaunchKernelGGL(row_mean_kernel<RT_DT_F32>, dim3((uint32_t)rows), dim3(kThreads), 0, stream,
-                               (uint64_t)g, row_len, inv_loss_scale, d_row_mean);
-            break;
-        case RT_DT_F16:
-            hipLaunchKernelGGL(row_mean_kernel<RT_DT_F16>, dim3((uint32_t)rows), dim3(kThreads), 0, stream,
-                               (uint64_t)g, row_len, inv_loss_scale, d_row_mean);
-            break;
-        default: return fail(RT_EINVAL, "g_dtype %d unknown", g_dtype);
+    if (row_len <= kWaveRowMax) {
+        const uint32_t grid = (uint32_t)((rows + kThreads / 64 - 1) / (kThreads / 64));
+        hipLaunchKernelGGL(row_mean_kernel, dim3(grid), dim3(kThreads), 0, stream, (uint64_t)g, (uint32_t)g_dtype, rows,
+                           (uint32_t)row_len, inv_loss_scale, d_row_mean);
+    } else {
+        hipLaunchKernelGGL(row_mean_long_kernel, dim3((uint32_t)rows), dim3(kThreads), 0, stream, (uint64_t)g,
+                           (uint32_t)g_dtype, row_len, inv_loss_scale, d_row_mean);
     }
     HIP_TRY(hipGetLastError());
     return RT_OK;
@@ -992,9 +987,11 @@ int rt_row_means_multi(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, fl
     if (n > 0 && !descs) return fail(RT_EINVAL, "descs is NULL");
     hipStream_t stream = (hipStream_t)stream_;
     HIP_TRY(hipSetDevice(h->device));
+    // Two tables, one per kernel: gradients whose rows one wavefront sums, and gradients with longer rows.
     std::vector<RowMeanEntry>& tab = h->rowmean_table;
     tab.clear();
-    uint64_t rows_total = 0;
+    std::vector<RowMeanEntry> long_tab;
+    uint64_t rows_short = 0, rows_long = 0;
     for (uint32_t i = 0; i < n; ++i) {
         const rt_tensor_desc& d = descs[i];
         if (d.numel == 0 || !d.row_mean) continue;
@@ -1004,27 +1001,49 @@ int rt_row_means_multi(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, fl
         if (d.g_dtype > RT_DT_F16) return fail(RT_EINVAL, "tensor %u: g_dtype %d (need bf16, f32 or f16)", i, d.g_dtype);
         if (d.host_mask & RT_HOST_G) return fail(RT_EINVAL, "tensor %u: the gradient must be device resident", i);
         if ((uintptr_t)d.g % dtype_size(d.g_dtype)) return fail(RT_EINVAL, "tensor %u: gradient pointer not aligned", i);
+        const bool is_long = d.row_len > kWaveRowMax;
+        uint64_t& rows = is_long ? rows_long : rows_short;
         RowMeanEntry e;
         e.g = (uint64_t)d.g;
         e.out = (uint64_t)d.row_mean;
         e.row_len = d.row_len;
-        e.first_row = (uint32_t)rows_total;
+        e.first_row = (uint32_t)rows;
         e.dtype = (uint32_t)d.g_dtype;
-        tab.push_back(e);
-        rows_total += d.numel / d.row_len;
-        if (rows_total > kMaxGrid) return fail(RT_EUNSUPPORTED, "more than %llu rows in one call", (unsigned long long)kMaxGrid);
+        (is_long ? long_tab : tab).push_back(e);
+        rows += d.numel / d.row_len;
+        if (rows > kMaxGrid) return fail(RT_EUNSUPPORTED, "more than %llu rows in one call", (unsigned long long)kMaxGrid);
     }
-    if (rows_total == 0) return RT_OK;
-    // the table goes through a staging slot, like the tables of the update
+    if (rows_short + rows_long == 0) return RT_OK;
+    // image: [first rows, short][records, short][first rows, long][records, long]; through a staging slot, like
+    // the tables of the update (the same gradients step after step upload nothing)
+    const size_t ns = tab.size(), nl = long_tab.size();
+    const size_t off_rec_s = align_up(ns * sizeof(uint32_t), 128);
+    const size_t off_first_l = off_rec_s + align_up(ns * sizeof(RowMeanEntry), 128);
+    const size_t off_rec_l = off_first_l + align_up(nl * sizeof(uint32_t), 128);
     Plan plan;
-    plan.bytes = tab.size() * sizeof(RowMeanEntry);
-    h->image.assign((const uint8_t*)tab.data(), (const uint8_t*)tab.data() + plan.bytes);
+    plan.bytes = off_rec_l + align_up(nl * sizeof(RowMeanEntry), 128);
+    h->image.assign(plan.bytes, 0);
+    uint8_t* img = h->image.data();
+    for (size_t k = 0; k < ns; ++k) ((uint32_t*)img)[k] = tab[k].first_row;
+    if (ns) memcpy(img + off_rec_s, tab.data(), ns * sizeof(RowMeanEntry));
+    for (size_t k = 0; k < nl; ++k) ((uint32_t*)(img + off_first_l))[k] = long_tab[k].first_row;
+    if (nl) memcpy(img + off_rec_l, long_tab.data(), nl * sizeof(RowMeanEntry));
     TableSlot* slot = nullptr;
-    int rc = stage_image(h, plan, h->image.data(), 0, stream, &slot);
+    int rc = stage_image(h, plan, img, 0, stream, &slot);
     if (rc != RT_OK) return rc;
-    hipLaunchKernelGGL(row_mean_table_kernel, dim3((uint32_t)rows_total), dim3(kThreads), 0, stream,
-                       (const RowMeanEntry*)slot->dev.ptr, (uint32_t)tab.size(), inv_loss_scale);
-    HIP_TRY(hipGetLastError());
+    const uint8_t* dev = (const uint8_t*)slot->dev.ptr;
+    if (rows_short) {
+        const uint32_t grid = (uint32_t)((rows_short + kThreads / 64 - 1) / (kThreads / 64));
+        hipLaunchKernelGGL(row_mean_table_kernel, dim3(grid), dim3(kThreads), 0, stream, (const uint32_t*)dev,
+                           (const RowMeanEntry*)(dev + off_rec_s), (uint32_t)ns, (uint32_t)rows_short, inv_loss_scale);
+        HIP_TRY(hipGetLastError());
+    }
+    if (rows_long) {
+        hipLaunchKernelGGL(row_mean_table_long_kernel, dim3((uint32_t)rows_long), dim3(kThreads), 0, stream,
+                           (const uint32_t*)(dev + off_first_l), (const RowMeanEntry*)(dev + off_rec_l), (uint32_t)nl,
+                           inv_loss_scale);
+        HIP_TRY(hipGetLastError());
+    }
     HIP_TRY(hipEventRecord(slot->done, stream));
     slot->in_flight = true;
     return RT_OK;

@@ -528,7 +528,8 @@ __global__ __launch_bounds__(kThreads) void sr_adamw_fast_kernel(const LaunchArg
     // a vector leave as its arithmetic finishes (holding them back to the end of the unit costs 60
     // registers and 0.4 %).  Against keeping one vector ahead this measured
     // 0.3 - 0.4 % faster on the 8B set, 5 % on a single 4096 x 4096 tensor and on the set of 20 064
-    // small tensors, at 99 vector registers instead of 68.
+    // small tensors, at 99 vector registers instead of 68 (explicit-noise instance: 159, and still 2 %
+    // faster on the single tensor than with one or two vectors ahead).
     In q[kFastIters];
     auto advance = [&]() {
         if constexpr (CEN) {
@@ -1285,33 +1286,112 @@ __global__ __launch_bounds__(kThreads) void grad_norm_finish_kernel(const double
     }
 }
 
-// Row means for centralization: one workgroup per row.  The sum of one row, in every thread:
+// ---------------------------------------------------------------------------
+// Row means for centralization (adamw.py:179-184).  A pure read of the gradients, 2 or 4 bytes per
+// element, so what matters is how many loads are in flight:
+//  * rows of at most kWaveRowMax elements (every matrix of a transformer) are summed by ONE
+//    wavefront each.  A lane issues up to eight 128-bit loads (sixteen for fp32) before its first
+//    add, each load instruction contiguous across the wave; no LDS, no barrier, and the four waves
+//    of a workgroup work on four rows independently;
+//  * longer rows (a huge 1-D tensor is a single row) take one workgroup per row, four vectors per
+//    thread in flight, and one LDS reduction per row.
+// Which of the two a row takes depends on its length alone, and both entry points (one gradient, or
+// the gradients of a whole step through a table) use the same two functions, so the same row
+// gives the same bits through either.
+// ---------------------------------------------------------------------------
+constexpr uint32_t kWaveRowMax = 32768;
+constexpr int kRowVecs = 8;   // vectors of 8 elements per lane and batch of the wave path
+
 template <int GDT>
-__device__ __forceinline__ float row_sum(uint64_t g, uint64_t base, uint64_t row_len, float inv_loss_scale, float* lds) {
-    const bool aligned = (g & 15u) == 0 && (row_len % kVec) == 0;
-    float acc = 0.0f;
-    for (uint64_t c = (uint64_t)threadIdx.x * kVec; c < row_len; c += (uint64_t)kThreads * kVec) {
-        const bool full = aligned && (c + kVec <= row_len);
-        const Raw8<GDT> r = full ? load_raw<GDT>(g, base + c) : load_raw_guarded<GDT>(g, base + c, base + row_len);
-        float x[8];
-        decode<GDT>(r, x);
+__device__ __forceinline__ float add_vec(float acc, const Raw8<GDT>& r, float inv_loss_scale) {
+    float x[8];
+    decode<GDT>(r, x);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc = acc + x[j] * inv_loss_scale;
+    for (int j = 0; j < 8; ++j) acc = acc + x[j] * inv_loss_scale;
+    return acc;
+}
+
+// Sum of row [base, base + row_len) of g by the calling wavefront; the result is in every lane.
+template <int GDT>
+__device__ __forceinline__ float row_sum_wave(uint64_t g, uint64_t base, uint32_t row_len, float inv_loss_scale) {
+    const uint32_t lane = threadIdx.x & 63u;
+    const bool aligned = ((g + base * esize<GDT>()) & 15u) == 0;   // vectors start at multiples of 8 elements of the row
+    float acc = 0.0f;
+    for (uint32_t c0 = 0; c0 < row_len; c0 += 64u * kVec * kRowVecs) {
+        Raw8<GDT> r[kRowVecs];
+#pragma unroll
+        for (int k = 0; k < kRowVecs; ++k) {
+            const uint32_t e = c0 + ((uint32_t)k * 64u + lane) * kVec;
+            if (e < row_len)
+                r[k] = (aligned && e + kVec <= row_len) ? load_raw<GDT>(g, base + e)
+                                                        : load_raw_guarded<GDT>(g, base + e, base + row_len);
+        }
+#pragma unroll
+        for (int k = 0; k < kRowVecs; ++k) {
+            const uint32_t e = c0 + ((uint32_t)k * 64u + lane) * kVec;
+            if (e < row_len) acc = add_vec<GDT>(acc, r[k], inv_loss_scale);
+        }
+    }
+    return wave_sum(acc);
+}
+
+// Sum of one (long) row by the calling workgroup; valid in thread 0.
+template <int GDT>
+__device__ __forceinline__ float row_sum_block(uint64_t g, uint64_t base, uint64_t row_len, float inv_loss_scale,
+                                               float* lds) {
+    constexpr int kInFlight = 4;
+    const bool aligned = ((g + base * esize<GDT>()) & 15u) == 0;
+    float acc = 0.0f;
+    for (uint64_t c0 = 0; c0 < row_len; c0 += (uint64_t)kThreads * kVec * kInFlight) {
+        Raw8<GDT> r[kInFlight];
+#pragma unroll
+        for (int k = 0; k < kInFlight; ++k) {
+            const uint64_t e = c0 + ((uint64_t)k * kThreads + threadIdx.x) * kVec;
+            if (e < row_len)
+                r[k] = (aligned && e + kVec <= row_len) ? load_raw<GDT>(g, base + e)
+                                                        : load_raw_guarded<GDT>(g, base + e, base + row_len);
+        }
+#pragma unroll
+        for (int k = 0; k < kInFlight; ++k) {
+            const uint64_t e = c0 + ((uint64_t)k * kThreads + threadIdx.x) * kVec;
+            if (e < row_len) acc = add_vec<GDT>(acc, r[k], inv_loss_scale);
+        }
     }
     return block_sum(acc, lds);
 }
 
-template <int GDT>
-__global__ __launch_bounds__(kThreads) void row_mean_kernel(uint64_t g, uint64_t row_len, float inv_loss_scale,
-                                                            float* __restrict__ out) {
+__device__ __forceinline__ float row_sum_wave_dt(uint32_t dt, uint64_t g, uint64_t base, uint32_t row_len, float inv) {
+    if (dt == RT_DT_BF16) return row_sum_wave<RT_DT_BF16>(g, base, row_len, inv);
+    if (dt == RT_DT_F32) return row_sum_wave<RT_DT_F32>(g, base, row_len, inv);
+    return row_sum_wave<RT_DT_F16>(g, base, row_len, inv);
+}
+__device__ __forceinline__ float row_sum_block_dt(uint32_t dt, uint64_t g, uint64_t base, uint64_t row_len, float inv,
+                                                  float* lds) {
+    if (dt == RT_DT_BF16) return row_sum_block<RT_DT_BF16>(g, base, row_len, inv, lds);
+    if (dt == RT_DT_F32) return row_sum_block<RT_DT_F32>(g, base, row_len, inv, lds);
+    return row_sum_block<RT_DT_F16>(g, base, row_len, inv, lds);
+}
+
+// One gradient.  Rows of at most kWaveRowMax elements: workgroup b takes rows 4b .. 4b+3, one per wave.
+__global__ __launch_bounds__(kThreads) void row_mean_kernel(uint64_t g, uint32_t dtype, uint64_t rows, uint32_t row_len,
+                                                            float inv_loss_scale, float* __restrict__ out) {
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const uint64_t row = (uint64_t)blockIdx.x * (kThreads / 64) + wave;
+    if (row >= rows) return;
+    const float sum = row_sum_wave_dt(dtype, g, row * row_len, row_len, inv_loss_scale);
+    if ((threadIdx.x & 63u) == 0) out[row] = sum / (float)row_len;
+}
+// Longer rows: one workgroup per row.
+__global__ __launch_bounds__(kThreads) void row_mean_long_kernel(uint64_t g, uint32_t dtype, uint64_t row_len,
+                                                                 float inv_loss_scale, float* __restrict__ out) {
     __shared__ float lds[kThreads / 64];
     const uint64_t row = blockIdx.x;
-    const float sum = row_sum<GDT>(g, row * row_len, row_len, inv_loss_scale, lds);
+    const float sum = row_sum_block_dt(dtype, g, row * row_len, row_len, inv_loss_scale, lds);
     if (threadIdx.x == 0) out[row] = sum / (float)row_len;
 }
 
-// The same for many gradients in one launch: workgroup b takes row b of the rows of all gradients
-// counted through, and finds its gradient by binary search over the first-row numbers.
+// The same for many gradients in one launch.  Rows are counted through all gradients of the launch;
+// `first` holds every gradient's first row number (ascending), `table` its record at the same index.
 struct alignas(16) RowMeanEntry {
     uint64_t g;
     uint64_t out;        // fp32[rows] of this gradient
@@ -1321,21 +1401,28 @@ struct alignas(16) RowMeanEntry {
 };
 static_assert(sizeof(RowMeanEntry) == 32, "RowMeanEntry layout");
 
-__global__ __launch_bounds__(kThreads) void row_mean_table_kernel(const RowMeanEntry* __restrict__ table, uint32_t n,
-                                                                  float inv_loss_scale) {
+__global__ __launch_bounds__(kThreads) void row_mean_table_kernel(const uint32_t* __restrict__ first,
+                                                                  const RowMeanEntry* __restrict__ table, uint32_t n,
+                                                                  uint32_t rows_total, float inv_loss_scale) {
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const uint32_t row = blockIdx.x * (kThreads / 64) + wave;
+    if (row >= rows_total) return;
+    const uint32_t idx = find_range(first, n, row);   // each wave searches on its own
+    const RowMeanEntry e = load_const(&table[idx]);
+    const uint64_t r = row - e.first_row;
+    const float sum = row_sum_wave_dt(e.dtype, e.g, r * e.row_len, (uint32_t)e.row_len, inv_loss_scale);
+    if ((threadIdx.x & 63u) == 0) ((RT_GLOBAL float*)e.out)[r] = sum / (float)e.row_len;
+}
+
+__global__ __launch_bounds__(kThreads) void row_mean_table_long_kernel(const uint32_t* __restrict__ first,
+                                                                       const RowMeanEntry* __restrict__ table, uint32_t n,
+                                                                       float inv_loss_scale) {
     __shared__ float lds[kThreads / 64];
     const uint32_t row = blockIdx.x;
-    uint32_t lo = 0, hi = n;  // the entry with the largest first_row <= row
-    while (hi - lo > 1) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (table[mid].first_row <= row) lo = mid; else hi = mid;
-    }
-    const RowMeanEntry e = table[lo];
+    const uint32_t idx = find_range(first, n, row);
+    const RowMeanEntry e = load_const(&table[idx]);
     const uint64_t r = row - e.first_row;
-    float sum;
-    if (e.dtype == RT_DT_BF16) sum = row_sum<RT_DT_BF16>(e.g, r * e.row_len, e.row_len, inv_loss_scale, lds);
-    else if (e.dtype == RT_DT_F32) sum = row_sum<RT_DT_F32>(e.g, r * e.row_len, e.row_len, inv_loss_scale, lds);
-    else sum = row_sum<RT_DT_F16>(e.g, r * e.row_len, e.row_len, inv_loss_scale, lds);
+    const float sum = row_sum_block_dt(e.dtype, e.g, r * e.row_len, e.row_len, inv_loss_scale, lds);
     if (threadIdx.x == 0) ((RT_GLOBAL float*)e.out)[r] = sum / (float)e.row_len;
 }
 

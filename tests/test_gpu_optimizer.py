@@ -326,7 +326,7 @@ def test_optimizer_with_loss_scale_and_max_grad_norm():
 
 
 @pytest.mark.parametrize("shape", [(37, 24), (4, 3, 10), (129,), (), (64, 300), (3000, 8), (5, 4099), (16, 1024, 3),
-                                   (20_000,), (4, 8192), (2500, 7)])
+                                   (20_000,), (4, 8192), (2500, 7), (2, 40_000), (70_001,), (3, 32_768), (3, 32_769)])
 def test_centralization(shape):
     n = int(np.prod(shape)) if len(shape) else 1
     p, g, _, _ = oracle.synth_inputs(n, 800)
@@ -375,12 +375,13 @@ def test_centralization_in_pieces_equals_whole(shape):
 
 def test_row_means_of_many_gradients_in_one_launch():
     """rt_row_means_multi = rt_row_means tensor by tensor, bit for bit (same summation), for row
-    lengths around the vector width, unaligned views and every gradient dtype."""
+    lengths around the vector width and on both sides of the length from which a row takes a whole
+    workgroup, unaligned views and every gradient dtype."""
     rng = np.random.default_rng(11)
     h = N.Handle(0)
     jobs, singles = [], []
     for k in range(40):
-        row_len = int(rng.choice([1, 3, 8, 12, 100, 511, 4096, 5000]))
+        row_len = int(rng.choice([1, 3, 8, 12, 100, 511, 4096, 5000, 32_768, 33_001, 70_001]))   # one wavefront per row up to 32 768 elements, a workgroup beyond
         rows = int(rng.integers(1, 40))
         dt = [torch.bfloat16, torch.float32, torch.float16][k % 3]
         off = int(rng.integers(0, 3))                     # a view that does not start on 16 bytes
