@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define RT_ABI_VERSION 2
+#define RT_ABI_VERSION 3
 
 /* error codes */
 #define RT_OK 0
@@ -144,20 +144,25 @@ int rt_step_multi(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const r
  * d_clip_coef / d_skip: as for rt_step_multi (device pointers, may be NULL);
  * they must be final for work queued on `stream` before the call.
  * Ordering against `stream`: the update kernels always wait for the work queued
- * on it.  The uploads wait for it only for tensors whose gradient lies in pinned
- * host memory (an asynchronous device-to-host copy on `stream` may still be
- * filling it, as after grad.to("cpu", non_blocking=True)) or that carry
- * RT_HOST_ORDERED; host-resident p / m / v are otherwise taken to be final in
- * host memory when the call is made (they are the optimizer's own to write).
- * Host arrays need not be pinned: the gradients that ramtorch's Linear.backward
- * leaves in ordinary CPU memory (linear.py:416-427, shipped up at adamw.py:167)
- * are copied into pinned bounce buffers of the handle (4 per array, one chunk
- * each) by a few host threads while earlier chunks are on the link, and the
- * call then hands the pipeline one chunk at a time.  RT_STREAM_BOUNCE_THREADS
- * in the environment sets the number of threads (default 4; 0 leaves such
- * copies to the runtime, which stages them while the calling thread waits).
- * Updated arrays that go back into memory that is not pinned are always left
- * to the runtime.
+ * on it.  This call, which returns only when everything is done, also waits
+ * for `stream` on the host before it uploads anything (unless an asynchronous
+ * call on the handle is still running), so whatever that work writes into host
+ * arrays -- a gradient copied down with grad.to("cpu", non_blocking=True), a
+ * parameter refreshed with p.copy_(gpu_tensor, non_blocking=True) -- is final.
+ * rt_step_streamed_async cannot wait on the host: there the uploads wait for
+ * `stream` only for tensors whose gradient lies in pinned host memory or that
+ * carry RT_HOST_ORDERED, and host-resident p / m / v are otherwise taken to be
+ * final in host memory when the call is made.
+ * Host arrays need not be pinned (plain CPU tensors, adamw.py:152-170; the
+ * gradients that ramtorch's Linear.backward leaves in ordinary CPU memory,
+ * linear.py:416-427, shipped up at adamw.py:167): on the way up they are
+ * copied into pinned bounce buffers of the handle (4 per array, one chunk
+ * each) by a few host threads while earlier chunks are on the link, on the way
+ * down (updated p / m / v, adamw.py:204-222) they land in such buffers and the
+ * threads copy them out, and the call hands the pipeline one chunk at a time.
+ * RT_STREAM_BOUNCE_THREADS in the environment sets the number of threads
+ * (default 8; 0 leaves such copies to the runtime, which stages them while the
+ * calling thread waits).
  */
 int rt_step_streamed(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, const rt_scalars* scalars,
                      uint32_t n_scalars, uint64_t seed, int noise_mode, uint64_t chunk_elems,
@@ -195,6 +200,53 @@ int rt_streamed_plan(const rt_tensor_desc* descs, uint32_t n, uint64_t chunk_ele
                      uint32_t* n_out);
 
 /*
+ * The order of operations of a streamed call, without touching a GPU: what the
+ * library itself executes for a call over n_chunks chunks, one rt_sched_op per
+ * operation in the order the host issues them.  The reference keeps its own
+ * staging buffers apart with ping-pong buffers and events
+ * (ramtorch/modules/linear.py:163-197, 267-308) and full-device syncs
+ * (adamw.py:227-232); here the discipline is this list, and it can be replayed
+ * on a CPU under any interleaving of the three streams to check that no
+ * staging or bounce buffer is written while something still reads it.
+ *   seq0:         chunks the handle has processed before this call (chunk c
+ *                 uses staging buffer (seq0 + c) % 2 and bounce slot (seq0 + c) % 4)
+ *   used_mask:    bit b set: staging buffer b holds a chunk of an earlier call
+ *                 whose download the first upload into it must await
+ *   paced_up:     some uploaded host array is not pinned (goes up through bounce slots)
+ *   paced_down:   some updated host array is not pinned (comes down through bounce slots)
+ *   batch_chunks: chunks queued at once when nothing is paced (0 = all)
+ * *n_out receives the number of operations; at most `cap` are written to `out`
+ * (may be NULL).
+ */
+enum {
+    RT_OP_HOST_WAIT_BACK = 0, /* host sleeps until `value` chunks have come back (a counter published behind each) */
+    RT_OP_HOST_FILL = 1,      /* host threads start copying chunk's unpinned arrays into upload bounce slot `bounce` */
+    RT_OP_HOST_WAIT_FILL = 2, /* host waits until those copies are done */
+    RT_OP_HOST_DRAIN = 3,     /* host threads start copying chunk's results out of download bounce slot `bounce` */
+    RT_OP_HOST_WAIT_DRAIN = 4,/* host waits until those copies are done */
+    RT_OP_H2D = 5,            /* upload stream: host arrays (or upload slot `bounce`) -> staging buffer `stage` */
+    RT_OP_KERNEL = 6,         /* compute stream: update in staging buffer `stage` */
+    RT_OP_D2H = 7,            /* download stream: staging buffer `stage` -> host arrays (or download slot `bounce`) */
+    RT_OP_PUBLISH = 8,        /* download stream: the chunk counter becomes `value` */
+    RT_OP_TICKET = 9,         /* download stream: the call's ticket is published */
+    RT_OP_HOST_WAIT_IDLE = 10 /* host waits until every earlier call on the handle has finished (a paced call starts
+                                 with it: the bounce slots and the chunk counter are shared with those calls) */
+};
+enum { RT_EV_H2D_DONE = 0, RT_EV_COMP_DONE = 2, RT_EV_D2H_DONE = 4 }; /* + staging buffer index */
+#define RT_SCHED_NONE 0xFFFFFFFFu
+typedef struct rt_sched_op {
+    uint32_t kind;         /* RT_OP_* */
+    uint32_t chunk;        /* chunk of the call the operation belongs to */
+    uint32_t stage;        /* staging buffer, or RT_SCHED_NONE */
+    uint32_t bounce;       /* bounce slot, or RT_SCHED_NONE */
+    uint32_t wait_event;   /* stream operations: event waited for before it starts, or RT_SCHED_NONE */
+    uint32_t record_event; /* stream operations: event recorded behind it, or RT_SCHED_NONE */
+    uint64_t value;        /* RT_OP_HOST_WAIT_BACK, RT_OP_PUBLISH */
+} rt_sched_op;
+int rt_streamed_schedule(uint32_t n_chunks, uint64_t seq0, uint32_t used_mask, int paced_up, int paced_down,
+                         uint64_t batch_chunks, rt_sched_op* out, uint32_t cap, uint32_t* n_out);
+
+/*
  * Global gradient norm over n device tensors (uses g, g_dtype, numel of each
  * desc), for the optional clip / skip check; not in the reference.  Writes to
  * d_out (device, 16-byte aligned):
@@ -216,9 +268,12 @@ int rt_grad_norm(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, float in
  * GPU, held until the process ends), the table travels there as kernel
  * arguments, and the call performs no hipMalloc / hipFree / hipHostMalloc.
  * Limit: at most 4096 gradients with numel != 0 per call; more returns
- * RT_EUNSUPPORTED.  Every call on one GPU uses that GPU's one array: calls
- * that overlap on a GPU (different streams or handles) race; calls queued on
- * one stream are safe.
+ * RT_EUNSUPPORTED.  Every call on one GPU uses that GPU's one array.  Outside
+ * stream capture the calls take turns on the GPU, whichever handle or stream
+ * they come from: each waits for an event recorded behind the previous one
+ * (the event exists since rt_create; nothing is allocated per call).  Under
+ * stream capture no event is used, and replays of graphs that contain such
+ * calls race if they overlap on a GPU: their owner has to order them.
  */
 int rt_grad_norm_static(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, float inv_loss_scale,
                         float max_norm, void* d_out, void* stream);

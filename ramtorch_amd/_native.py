@@ -15,7 +15,7 @@ import weakref
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "_lib", "libramtorch_sr_adamw.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 RT_OK = 0
 RT_EINVAL, RT_EHIP, RT_ENOMEM, RT_EUNSUPPORTED = -1, -2, -3, -4
@@ -31,7 +31,7 @@ EXPORTS = (
     "rt_stream_probe", "rt_streamed_timeline", "rt_streamed_plan",
     "rt_step_streamed_async", "rt_streamed_wait", "rt_streamed_completed",
     "rt_grad_norm_static", "rt_host_link_probe", "rt_selftest_sqrt", "rt_dev_hold", "rt_dev_release",
-    "rt_streamed_bounce_stats", "rt_row_means_multi",
+    "rt_streamed_bounce_stats", "rt_row_means_multi", "rt_streamed_schedule",
 )
 
 
@@ -80,6 +80,25 @@ class RtTensorDesc(ctypes.Structure):
     ]
 
 
+class RtSchedOp(ctypes.Structure):
+    """One operation of a streamed call's schedule (``rt_sched_op``)."""
+    _fields_ = [
+        ("kind", ctypes.c_uint32),
+        ("chunk", ctypes.c_uint32),
+        ("stage", ctypes.c_uint32),
+        ("bounce", ctypes.c_uint32),
+        ("wait_event", ctypes.c_uint32),
+        ("record_event", ctypes.c_uint32),
+        ("value", ctypes.c_uint64),
+    ]
+
+
+(RT_OP_HOST_WAIT_BACK, RT_OP_HOST_FILL, RT_OP_HOST_WAIT_FILL, RT_OP_HOST_DRAIN, RT_OP_HOST_WAIT_DRAIN, RT_OP_H2D,
+ RT_OP_KERNEL, RT_OP_D2H, RT_OP_PUBLISH, RT_OP_TICKET, RT_OP_HOST_WAIT_IDLE) = range(11)
+RT_EV_H2D_DONE, RT_EV_COMP_DONE, RT_EV_D2H_DONE = 0, 2, 4
+RT_SCHED_NONE = 0xFFFFFFFF
+
+assert ctypes.sizeof(RtSchedOp) == 32
 assert ctypes.sizeof(RtScalars) == 48
 assert ctypes.sizeof(RtTensorDesc) == 136
 
@@ -155,6 +174,8 @@ def lib() -> ctypes.CDLL:
     L.rt_streamed_completed.argtypes = [vp, ctypes.POINTER(u64)]
     L.rt_streamed_plan.restype = i32
     L.rt_streamed_plan.argtypes = [descs, u32, u64, ctypes.POINTER(u64), u32, ctypes.POINTER(u32)]
+    L.rt_streamed_schedule.restype = i32
+    L.rt_streamed_schedule.argtypes = [u32, u64, u32, i32, i32, u64, ctypes.POINTER(RtSchedOp), u32, ctypes.POINTER(u32)]
     L.rt_streamed_stats.restype = i32
     L.rt_streamed_stats.argtypes = [vp, ctypes.POINTER(ctypes.c_double)]
     L.rt_streamed_bounce_stats.restype = i32
@@ -347,6 +368,18 @@ def streamed_plan(descs, n: int, chunk_elems: int):
     buf = (ctypes.c_uint64 * max(5 * k.value, 1))()
     check(lib().rt_streamed_plan(descs, n, chunk_elems, buf, k.value, ctypes.byref(k)))
     return [tuple(buf[5 * i:5 * i + 5]) for i in range(k.value)]
+
+
+def streamed_schedule(n_chunks: int, seq0: int = 0, used_mask: int = 0, paced_up: bool = False,
+                      paced_down: bool = False, batch_chunks: int = 64):
+    """The operations of a streamed call in the order the host issues them (host only): a list of
+    ``RtSchedOp``.  This is the list the library itself executes."""
+    k = ctypes.c_uint32()
+    args = (int(n_chunks), int(seq0), int(used_mask), int(paced_up), int(paced_down), int(batch_chunks))
+    check(lib().rt_streamed_schedule(*args, None, 0, ctypes.byref(k)))
+    buf = (RtSchedOp * max(k.value, 1))()
+    check(lib().rt_streamed_schedule(*args, buf, k.value, ctypes.byref(k)))
+    return list(buf[:k.value])
 
 
 def dev_release(addr: int) -> None:

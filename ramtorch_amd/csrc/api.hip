@@ -118,8 +118,12 @@ struct Streamed {
     // host threads fill while earlier chunks are on the link; see streamed_enqueue_impl.
     void* bounce[4][kBounce] = {};
     size_t bounce_cap[4] = {0, 0, 0, 0};   // bytes of each of the kBounce buffers of an array
+    // The same for the way back: updated p / m / v that belong into host memory that is not pinned land in
+    // these and host threads copy them out (index 1, the gradient, stays unused).
+    void* bounce_down[4][kBounce] = {};
+    size_t bounce_down_cap[4] = {0, 0, 0, 0};
     std::unique_ptr<CopyPool> pool;
-    int bounce_threads = 4;   // RT_STREAM_BOUNCE_THREADS in the environment overrides; 0 leaves such copies to the runtime
+    int bounce_threads = 8;   // RT_STREAM_BOUNCE_THREADS in the environment overrides; 0 leaves such copies to the runtime
     uint64_t paced_calls = 0, bounced_bytes = 0;
 };
 
@@ -174,6 +178,11 @@ constexpr int kMaxDevices = 64;
 }  // namespace
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 static void* g_scratch_ptr[kMaxDevices];  // device -> address of that device's copy of `scratch`
+// Every call on a device shares that device's array.  An event recorded behind the last call's kernels
+// lets the next call wait for them on the GPU, whichever handle or stream it comes from, so that calls
+// which would overlap take turns instead of racing.  (Not under stream capture: a graph's replays are its
+// owner's to order.)
+static hipEvent_t g_scratch_done[kMaxDevices];
 static std::mutex g_scratch_mutex;
 
 struct rt_handle {
@@ -730,6 +739,7 @@ int rt_create(int device, rt_handle** out) {
         if (!g_scratch_ptr[device]) {
             void* ptr = nullptr;
             HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));  // with `device` current: its own copy
+            HIP_TRY(hipEventCreateWithFlags(&g_scratch_done[device], hipEventDisableTiming));
             g_scratch_ptr[device] = ptr;
         }
         scratch_ptr = g_scratch_ptr[device];
@@ -783,8 +793,10 @@ int rt_destroy(rt_handle* h) {
     }
     st.pool.reset();  // joins the copy threads
     for (int a = 0; a < 4; ++a)
-        for (int k = 0; k < kBounce; ++k)
+        for (int k = 0; k < kBounce; ++k) {
             if (st.bounce[a][k]) (void)hipHostFree(st.bounce[a][k]);
+            if (st.bounce_down[a][k]) (void)hipHostFree(st.bounce_down[a][k]);
+        }
     if (st.ticket_word) (void)hipHostFree((void*)st.ticket_word);
     for (hipEvent_t e : st.tl_events) (void)hipEventDestroy(e);
     if (st.start) (void)hipEventDestroy(st.start);
@@ -938,6 +950,17 @@ int rt_grad_norm_static(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, f
     if (rc != RT_OK) return rc;
     double* partials = (double*)h->static_scratch;
     NormEntry* table = (NormEntry*)((uint8_t*)h->static_scratch + kStaticPartialsBytes);
+    // take turns with whatever call used the array last (nothing is allocated: the event exists since rt_create)
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) {
+        (void)hipGetLastError();
+        capturing = hipStreamCaptureStatusNone;
+    }
+    std::unique_lock<std::mutex> turn(g_scratch_mutex, std::defer_lock);
+    if (capturing == hipStreamCaptureStatusNone) {
+        turn.lock();   // wait-then-record is one step as seen by other host threads
+        HIP_TRY(hipStreamWaitEvent(stream, g_scratch_done[h->device], 0));
+    }
     const uint32_t n_chunks = (uint32_t)(n_whole + n_rest);
     const uint32_t grid = std::min<uint32_t>(kNormPartials, n_chunks);
     // the table reaches the device array as kernel arguments, a slice per launch
@@ -957,6 +980,7 @@ int rt_grad_norm_static(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, f
     hipLaunchKernelGGL(grad_norm_finish_kernel, dim3(1), dim3(kThreads), 0, stream, (const double*)partials, grid,
                        max_norm, (float*)d_out);
     HIP_TRY(hipGetLastError());
+    if (capturing == hipStreamCaptureStatusNone) HIP_TRY(hipEventRecord(g_scratch_done[h->device], stream));
     return RT_OK;
 }
 
@@ -1171,6 +1195,95 @@ int rt_streamed_plan(const rt_tensor_desc* descs, uint32_t n, uint64_t chunk_ele
     return RT_OK;
 }
 
+// ---------------------------------------------------------------------------
+// The order of everything a streamed call does, as data.  build_schedule lists, in the order the host
+// issues them, the operations of a call over n_chunks chunks: what runs on which stream, which
+// staging buffer and bounce slot it touches, which event it waits for and which it records, and where
+// the host itself waits.  streamed_enqueue_impl executes exactly this list, and rt_streamed_schedule
+// hands it out so that the discipline -- no staging or bounce buffer is written while something still
+// reads it or reads it before it has been written -- can be checked on a CPU by replaying the list
+// under arbitrary interleavings of the streams (tests/test_host.py).
+//
+//   H2D(c)    upload stream:  waits for D2H_DONE of the staging buffer's previous chunk, records H2D_DONE
+//   KERNEL(c) compute stream: waits for H2D_DONE, records COMP_DONE
+//   D2H(c)    download stream: waits for COMP_DONE, records D2H_DONE
+// Up front (everything pinned) the whole call is queued at once, in batches of `batch` chunks with a
+// drain in between.  Paced (some host array is not pinned) the host feeds the pipeline chunk by chunk:
+// chunk c goes onto the streams when chunk c - kPacedInFlight has come back (a counter the download
+// stream publishes behind every chunk), when host threads have filled its upload bounce slot, and when
+// the copies out of the download bounce slot it is going to reuse are done.
+// ---------------------------------------------------------------------------
+static void build_schedule(uint32_t n_chunks, uint64_t seq0, uint32_t used_mask, bool paced_up, bool paced_down,
+                           uint64_t batch, std::vector<rt_sched_op>& ops) {
+    ops.clear();
+    const bool paced = paced_up || paced_down;
+    bool used[kStageBufs];
+    for (int b = 0; b < kStageBufs; ++b) used[b] = (used_mask >> b) & 1u;
+    auto push = [&](uint32_t kind, uint32_t chunk, uint32_t stage, uint32_t bounce, uint32_t wait_ev, uint32_t rec_ev,
+                    uint64_t value) {
+        rt_sched_op op;
+        op.kind = kind; op.chunk = chunk; op.stage = stage; op.bounce = bounce;
+        op.wait_event = wait_ev; op.record_event = rec_ev; op.value = value;
+        ops.push_back(op);
+    };
+    const uint32_t none = RT_SCHED_NONE;
+    auto slot_of = [&](uint64_t c) { return (uint32_t)((seq0 + c) % kBounce); };
+    uint32_t fills_submitted = 0, drains_submitted = 0;
+    if (paced && n_chunks) push(RT_OP_HOST_WAIT_IDLE, 0, none, none, none, none, 0);
+    for (uint32_t c = 0; c < n_chunks; ++c) {
+        const uint32_t b = (uint32_t)((seq0 + c) % kStageBufs);
+        if (paced) {
+            if (c >= kPacedInFlight) {
+                push(RT_OP_HOST_WAIT_BACK, c - (uint32_t)kPacedInFlight, none, none, none, none, seq0 + c - kPacedInFlight + 1);
+                if (paced_down) {   // that chunk's results lie in its download bounce slot: copy them out
+                    push(RT_OP_HOST_DRAIN, c - (uint32_t)kPacedInFlight, none, slot_of(c - kPacedInFlight), none, none, 0);
+                    drains_submitted = c - (uint32_t)kPacedInFlight + 1;
+                }
+            }
+            if (paced_down && c >= (uint32_t)kBounce)   // the download slot of this chunk was chunk c - kBounce's
+                push(RT_OP_HOST_WAIT_DRAIN, c - (uint32_t)kBounce, none, slot_of(c - kBounce), none, none, 0);
+            if (paced_up) {
+                // chunk k may be copied into its upload slot once chunk k - kBounce has left it, which is
+                // known when that chunk has come back
+                const uint32_t last = std::min<uint64_t>((uint64_t)c + kBounce - kPacedInFlight, n_chunks - 1);
+                for (; fills_submitted <= last; ++fills_submitted)
+                    push(RT_OP_HOST_FILL, fills_submitted, none, slot_of(fills_submitted), none, none, 0);
+                push(RT_OP_HOST_WAIT_FILL, c, none, slot_of(c), none, none, 0);
+            }
+        } else if (c > 0 && batch > 0 && c % batch == 0) {
+            // a long call is queued in batches and the pipeline drains between them
+            push(RT_OP_PUBLISH, c - 1, none, none, none, none, seq0 + c);
+            push(RT_OP_HOST_WAIT_BACK, c - 1, none, none, none, none, seq0 + c);
+        }
+        push(RT_OP_H2D, c, b, paced_up ? slot_of(c) : none, used[b] ? RT_EV_D2H_DONE + b : none, RT_EV_H2D_DONE + b, 0);
+        push(RT_OP_KERNEL, c, b, none, RT_EV_H2D_DONE + b, RT_EV_COMP_DONE + b, 0);
+        push(RT_OP_D2H, c, b, paced_down ? slot_of(c) : none, RT_EV_COMP_DONE + b, RT_EV_D2H_DONE + b, 0);
+        used[b] = true;
+        if (paced) push(RT_OP_PUBLISH, c, none, none, none, none, seq0 + c + 1);
+    }
+    push(RT_OP_TICKET, n_chunks ? n_chunks - 1 : 0, none, none, none, none, 0);
+    if (paced_down) {
+        // the last chunks: wait for each, copy its results out, and wait for every copy still running
+        for (uint32_t c = drains_submitted; c < n_chunks; ++c) {
+            push(RT_OP_HOST_WAIT_BACK, c, none, none, none, none, seq0 + c + 1);
+            push(RT_OP_HOST_DRAIN, c, none, slot_of(c), none, none, 0);
+        }
+        for (uint32_t c = n_chunks > (uint32_t)kBounce ? n_chunks - kBounce : 0; c < n_chunks; ++c)
+            push(RT_OP_HOST_WAIT_DRAIN, c, none, slot_of(c), none, none, 0);
+    }
+}
+
+extern "C" int rt_streamed_schedule(uint32_t n_chunks, uint64_t seq0, uint32_t used_mask, int paced_up, int paced_down,
+                                    uint64_t batch_chunks, rt_sched_op* out, uint32_t cap, uint32_t* n_out) {
+    if (!n_out) return fail(RT_EINVAL, "n_out is NULL");
+    if (used_mask >> kStageBufs) return fail(RT_EINVAL, "used_mask names a staging buffer that does not exist");
+    std::vector<rt_sched_op> ops;
+    build_schedule(n_chunks, seq0, used_mask, paced_up != 0, paced_down != 0, batch_chunks, ops);
+    for (size_t i = 0; out && i < ops.size() && i < cap; ++i) out[i] = ops[i];
+    *n_out = (uint32_t)ops.size();
+    return RT_OK;
+}
+
 // Highest ticket whose copies have all landed: a plain read of pinned host memory.
 static inline uint64_t tickets_done(const Streamed& st) {
     return st.ticket_word ? __atomic_load_n((const uint64_t*)st.ticket_word, __ATOMIC_ACQUIRE) : 0;
@@ -1238,10 +1351,10 @@ static bool is_pinned_host(const void* p) {
 namespace {
 struct FillGuard {
     CopyPool* pool = nullptr;
-    CopyPool::Group* groups = nullptr;
-    size_t submitted = 0;
+    std::vector<CopyPool::Group*> started;   // groups with copies submitted
     ~FillGuard() {
-        for (size_t i = 0; pool && i < submitted; ++i) pool->wait(&groups[i]);
+        for (CopyPool::Group* g : started)
+            if (pool) pool->wait(g);
     }
 };
 }  // namespace
@@ -1329,34 +1442,39 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
         bool need[4] = {false, false, false, false};
         for (uint32_t i = 0; i < n; ++i)
             for (int a = 0; a < 4; ++a) need[a] |= (unpinned[i] >> a) & 1;
-        for (int a = 0; a < 4; ++a) {
-            const size_t want = max_used * (size_t)stage_esize[a];
-            if (!need[a] || want <= st.bounce_cap[a]) continue;
-            for (int k = 0; k < kBounce; ++k) {
-                if (st.bounce[a][k]) HIP_TRY(hipHostFree(st.bounce[a][k]));
-                st.bounce[a][k] = nullptr;
-            }
-            st.bounce_cap[a] = 0;
-            bool got_all = true;
-            for (int k = 0; k < kBounce && got_all; ++k) {
-                if (hipHostMalloc(&st.bounce[a][k], want, hipHostMallocDefault) != hipSuccess) {
-                    (void)hipGetLastError();
-                    st.bounce[a][k] = nullptr;
-                    got_all = false;
-                }
-            }
-            if (!got_all) {
-                // No pinned memory to be had (a locked-memory limit, say): this call leaves the unpinned
-                // copies to the runtime, which is slower but needs nothing from us.
+        // upload slots for every such array, download slots for the ones that are written (not the gradient)
+        for (int dir = 0; dir < 2 && paced; ++dir)
+            for (int a = 0; a < 4; ++a) {
+                if (dir == 1 && a == 1) continue;
+                void* (&slots)[kBounce] = dir == 0 ? st.bounce[a] : st.bounce_down[a];
+                size_t& cap = dir == 0 ? st.bounce_cap[a] : st.bounce_down_cap[a];
+                const size_t want = max_used * (size_t)stage_esize[a];
+                if (!need[a] || want <= cap) continue;
                 for (int k = 0; k < kBounce; ++k) {
-                    if (st.bounce[a][k]) (void)hipHostFree(st.bounce[a][k]);
-                    st.bounce[a][k] = nullptr;
+                    if (slots[k]) HIP_TRY(hipHostFree(slots[k]));
+                    slots[k] = nullptr;
                 }
-                paced = false;
-                break;
+                cap = 0;
+                bool got_all = true;
+                for (int k = 0; k < kBounce && got_all; ++k) {
+                    if (hipHostMalloc(&slots[k], want, hipHostMallocDefault) != hipSuccess) {
+                        (void)hipGetLastError();
+                        slots[k] = nullptr;
+                        got_all = false;
+                    }
+                }
+                if (!got_all) {
+                    // No pinned memory to be had (a locked-memory limit, say): this call leaves the unpinned
+                    // copies to the runtime, which is slower but needs nothing from us.
+                    for (int k = 0; k < kBounce; ++k) {
+                        if (slots[k]) (void)hipHostFree(slots[k]);
+                        slots[k] = nullptr;
+                    }
+                    paced = false;
+                    break;
+                }
+                cap = want;
             }
-            st.bounce_cap[a] = want;
-        }
         if (paced) {
             ++st.paced_calls;
         } else {
@@ -1451,13 +1569,12 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
                        ((d.host_mask & RT_HOST_G) != 0 && !(unpinned_probe[i] & RT_HOST_G));
     }
     HIP_TRY(hipEventRecord(st.start, user));
-    if (upload_waits) {
-        // A call that returns only when everything is done, with nothing of the pipeline running
-        // yet, may as well wait on the host: even one such wait on the upload stream per call was
-        // measured to cost most calls the same 50 ms.
-        if (blocking && !st.pending) HIP_TRY(hipStreamSynchronize(user));
-        else HIP_TRY(hipStreamWaitEvent(st.h2d, st.start, 0));
-    }
+    // A call that returns only when everything is done, with nothing of the pipeline running yet,
+    // waits for the caller's stream on the host, whatever the tensors: it costs nothing (the call
+    // blocks anyway), it covers every way in which work on that stream may still be writing host
+    // arrays, and even one wait on the upload stream per call was measured to cost most calls 50 ms.
+    if (blocking && !st.pending) HIP_TRY(hipStreamSynchronize(user));
+    else if (upload_waits) HIP_TRY(hipStreamWaitEvent(st.h2d, st.start, 0));
     HIP_TRY(hipStreamWaitEvent(st.comp, st.start, 0));
     if (!blob.empty()) {
         const uint64_t n_vec = (blob.size() + 15) / 16;  // buffers are padded well past the blob
@@ -1477,123 +1594,123 @@ static int streamed_enqueue_impl(rt_handle* h, const rt_tensor_desc* descs, uint
             st.tl_events.push_back(e);
         }
     }
-    const uint64_t batch = st.batch_chunks;
-    std::unique_ptr<CopyPool::Group[]> fills(paced ? new CopyPool::Group[chunks.size()] : nullptr);
-    FillGuard guard;
+    // ---- the order of everything that follows is build_schedule's; this loop only carries it out
+    bool paced_up = false, paced_down = false;
+    for (uint32_t i = 0; i < n; ++i) {
+        paced_up |= unpinned[i] != 0;
+        paced_down |= (unpinned[i] & (RT_HOST_P | RT_HOST_M | RT_HOST_V)) != 0;
+    }
+    uint32_t used_mask = 0;
+    for (int b = 0; b < kStageBufs; ++b) used_mask |= st.used_buf[b] ? 1u << b : 0u;
+    std::vector<rt_sched_op> ops;
+    build_schedule((uint32_t)chunks.size(), st.seq, used_mask, paced_up, paced_down, st.batch_chunks, ops);
+    std::unique_ptr<CopyPool::Group[]> fills(paced_up ? new CopyPool::Group[chunks.size()] : nullptr);
+    std::unique_ptr<CopyPool::Group[]> drains(paced_down ? new CopyPool::Group[chunks.size()] : nullptr);
+    FillGuard guard;   // a call that leaves early waits for the copies already handed to the host threads
     guard.pool = st.pool.get();
-    guard.groups = fills.get();
-    // Chunk k may be copied into its bounce buffers once chunk k - kBounce has left them, which is
-    // known when that chunk's D2H has been published.
-    auto submit_fills_through = [&](size_t last) {
-        for (; guard.submitted <= last && guard.submitted < chunks.size(); ++guard.submitted) {
-            const size_t k = guard.submitted;
-            const int slot = (int)((st.seq + k) % kBounce);
-            for (const Segment& s : chunks[k]) {
-                const rt_tensor_desc& d = descs[s.tensor];
-                const uint8_t up = unpinned[s.tensor];
-                if (!up) continue;
-                const int es[4] = {dtype_size(d.p_dtype), dtype_size(d.g_dtype), dtype_size(d.m_dtype),
-                                   dtype_size(d.v_dtype)};
-                const void* host[4] = {d.p, d.g, d.m, d.v};
-                for (int a = 0; a < 4; ++a)
-                    if (up & (1u << a)) {
-                        st.pool->submit(&fills[k], (uint8_t*)st.bounce[a][slot] + s.stage_off * es[a],
-                                        (const uint8_t*)host[a] + s.start * es[a], s.count * es[a]);
-                        st.bounced_bytes += s.count * es[a];
-                    }
-            }
-        }
+    hipStream_t streams[3] = {st.h2d, st.comp, st.d2h};
+    auto event_of = [&](uint32_t id) -> hipEvent_t {
+        const uint32_t b = id & 1u;
+        return id < RT_EV_COMP_DONE ? st.h2d_done[b] : id < RT_EV_D2H_DONE ? st.comp_done[b] : st.d2h_done[b];
     };
-    for (size_t c = 0; c < chunks.size(); ++c) {
-        const int b = (int)((st.seq + c) % kStageBufs);
-        const auto& segs = chunks[c];
-        if (paced) {
-            // The host feeds the pipeline: chunk c goes onto the streams when chunk c - kPacedInFlight
-            // has come back (with a third chunk queued while two are on the streams the copies were
-            // measured at a third of their rate, also with three staging buffers per array),
-            // and when the host threads have filled its bounce buffers.  Every wait is a sleep on a
-            // word of pinned memory or on the pool's condition variable, never inside the runtime.
-            if (c >= kPacedInFlight && !sleep_until_word(st.ticket_word + 1, st.seq + c - kPacedInFlight + 1))
-                HIP_TRY(hipStreamSynchronize(st.d2h));  // stalled: block, and surface a device error
-            submit_fills_through(c + kBounce - kPacedInFlight);
-            st.pool->wait(&fills[c]);
-        }
-        // A long call is queued in batches, and the pipeline drains between them.  With a few
-        // hundred chunks waiting on the streams at once the copies of this pipeline were measured
-        // at well under half their rate, and queuing more while the streams are busy costs about
-        // as much; a drain costs one pipeline fill (about two chunk times) per batch.
-        if (!paced && c > 0 && c % batch == 0) {
-            hipLaunchKernelGGL(publish_ticket_kernel, dim3(1), dim3(1), 0, st.d2h,
-                               (uint64_t)(st.ticket_word + 1), st.seq + c);
-            HIP_TRY(hipGetLastError());
-            if (!sleep_until_word(st.ticket_word + 1, st.seq + c))
-                HIP_TRY(hipStreamSynchronize(st.d2h));  // stalled: block, and surface a device error
-        }
-        // H2D: the buffer is free once the D2H of the chunk that used it last has finished
-        if (st.used_buf[b]) HIP_TRY(hipStreamWaitEvent(st.h2d, st.d2h_done[b], 0));
-        if (trace) HIP_TRY(hipEventRecord(st.tl_events[4 * c + 0], st.h2d));
-        for (size_t k = 0; k < segs.size(); ++k) {
-            const Segment& s = segs[k];
-            const rt_tensor_desc& d = descs[s.tensor];
-            const int es[4] = {dtype_size(d.p_dtype), dtype_size(d.g_dtype), dtype_size(d.m_dtype),
-                               dtype_size(d.v_dtype)};
-            const void* host[4] = {d.p, d.g, d.m, d.v};
-            void* dev[4] = {pieces[c][k].p, (void*)pieces[c][k].g, pieces[c][k].m, pieces[c][k].v};
-            for (int a = 0; a < 4; ++a) {
-                if (!(d.host_mask & (1u << a))) continue;
-                const size_t bytes = s.count * es[a];
-                const uint8_t* src = (unpinned[s.tensor] & (1u << a))
-                                         ? (const uint8_t*)st.bounce[a][(st.seq + c) % kBounce] + s.stage_off * es[a]
-                                         : (const uint8_t*)host[a] + s.start * es[a];
-                HIP_TRY(hipMemcpyAsync(dev[a], src, bytes, hipMemcpyHostToDevice, st.h2d));
-                st.bytes_h2d += (double)bytes;
+    for (const rt_sched_op& op : ops) {
+        const size_t c = op.chunk;
+        switch (op.kind) {
+            case RT_OP_HOST_WAIT_BACK:
+                // Every wait is a sleep on a word of pinned memory, never inside the runtime.
+                if (!sleep_until_word(st.ticket_word + 1, op.value))
+                    HIP_TRY(hipStreamSynchronize(st.d2h));  // stalled: block, and surface a device error
+                break;
+            case RT_OP_HOST_FILL:
+            case RT_OP_HOST_DRAIN: {
+                const bool up = op.kind == RT_OP_HOST_FILL;
+                CopyPool::Group* grp = up ? &fills[c] : &drains[c];
+                guard.started.push_back(grp);
+                for (const Segment& sg : chunks[c]) {
+                    const rt_tensor_desc& d = descs[sg.tensor];
+                    const uint8_t mask = up ? unpinned[sg.tensor]
+                                            : (uint8_t)(unpinned[sg.tensor] & (RT_HOST_P | RT_HOST_M | RT_HOST_V));
+                    if (!mask) continue;
+                    const int es[4] = {dtype_size(d.p_dtype), dtype_size(d.g_dtype), dtype_size(d.m_dtype),
+                                       dtype_size(d.v_dtype)};
+                    void* host[4] = {d.p, (void*)d.g, d.m, d.v};
+                    for (int a = 0; a < 4; ++a)
+                        if (mask & (1u << a)) {
+                            uint8_t* user = (uint8_t*)host[a] + sg.start * es[a];
+                            uint8_t* slot = (uint8_t*)(up ? st.bounce[a] : st.bounce_down[a])[op.bounce] + sg.stage_off * es[a];
+                            if (up) st.pool->submit(grp, slot, user, sg.count * es[a]);
+                            else st.pool->submit(grp, user, slot, sg.count * es[a]);
+                            st.bounced_bytes += sg.count * es[a];
+                        }
+                }
+                break;
             }
-        }
-        if (trace) HIP_TRY(hipEventRecord(st.tl_events[4 * c + 1], st.h2d));
-        HIP_TRY(hipEventRecord(st.h2d_done[b], st.h2d));
-
-        // compute
-        HIP_TRY(hipStreamWaitEvent(st.comp, st.h2d_done[b], 0));
-        rc = enqueue_kernels(plans[c], (const uint8_t*)tab.dev.ptr + plan_off[c], seed, noise_mode, d_clip_coef,
-                             d_skip, st.comp);
-        if (rc != RT_OK) return rc;
-        HIP_TRY(hipEventRecord(st.comp_done[b], st.comp));
-
-        // D2H of the updated host-resident arrays (p, m, v; grads are read-only)
-        HIP_TRY(hipStreamWaitEvent(st.d2h, st.comp_done[b], 0));
-        if (trace) HIP_TRY(hipEventRecord(st.tl_events[4 * c + 2], st.d2h));
-        for (size_t k = 0; k < segs.size(); ++k) {
-            const Segment& s = segs[k];
-            const rt_tensor_desc& d = descs[s.tensor];
-            const int es[4] = {dtype_size(d.p_dtype), 0, dtype_size(d.m_dtype), dtype_size(d.v_dtype)};
-            void* host[4] = {d.p, nullptr, d.m, d.v};
-            const void* dev[4] = {pieces[c][k].p, nullptr, pieces[c][k].m, pieces[c][k].v};
-            for (int a = 0; a < 4; ++a) {
-                if (a == 1 || !(d.host_mask & (1u << a))) continue;
-                const size_t bytes = s.count * es[a];
-                HIP_TRY(hipMemcpyAsync((uint8_t*)host[a] + s.start * es[a], dev[a], bytes, hipMemcpyDeviceToHost,
-                                       st.d2h));
-                st.bytes_d2h += (double)bytes;
+            case RT_OP_HOST_WAIT_IDLE:
+                if (tickets_done(st) < st.tickets_issued) {
+                    rc = streamed_wait(h);
+                    if (rc != RT_OK) return rc;
+                    st.pending = true;   // this call's own work follows
+                }
+                break;
+            case RT_OP_HOST_WAIT_FILL: st.pool->wait(&fills[c]); break;
+            case RT_OP_HOST_WAIT_DRAIN: st.pool->wait(&drains[c]); break;
+            case RT_OP_H2D:
+            case RT_OP_D2H: {
+                const bool up = op.kind == RT_OP_H2D;
+                hipStream_t stream = up ? st.h2d : st.d2h;
+                if (op.wait_event != RT_SCHED_NONE) HIP_TRY(hipStreamWaitEvent(stream, event_of(op.wait_event), 0));
+                if (trace) HIP_TRY(hipEventRecord(st.tl_events[4 * c + (up ? 0 : 2)], stream));
+                const auto& segs = chunks[c];
+                for (size_t k = 0; k < segs.size(); ++k) {
+                    const Segment& sg = segs[k];
+                    const rt_tensor_desc& d = descs[sg.tensor];
+                    const int es[4] = {dtype_size(d.p_dtype), dtype_size(d.g_dtype), dtype_size(d.m_dtype),
+                                       dtype_size(d.v_dtype)};
+                    void* host[4] = {d.p, (void*)d.g, d.m, d.v};
+                    void* dev[4] = {pieces[c][k].p, (void*)pieces[c][k].g, pieces[c][k].m, pieces[c][k].v};
+                    for (int a = 0; a < 4; ++a) {
+                        if (!(d.host_mask & (1u << a)) || (!up && a == 1)) continue;   // gradients only go up
+                        const size_t bytes = sg.count * es[a];
+                        const bool bounced = (unpinned[sg.tensor] & (1u << a)) != 0;
+                        uint8_t* h_addr = bounced ? (uint8_t*)(up ? st.bounce[a] : st.bounce_down[a])[op.bounce] + sg.stage_off * es[a]
+                                                  : (uint8_t*)host[a] + sg.start * es[a];
+                        if (up) HIP_TRY(hipMemcpyAsync(dev[a], h_addr, bytes, hipMemcpyHostToDevice, stream));
+                        else HIP_TRY(hipMemcpyAsync(h_addr, dev[a], bytes, hipMemcpyDeviceToHost, stream));
+                        (up ? st.bytes_h2d : st.bytes_d2h) += (double)bytes;
+                    }
+                }
+                if (trace) HIP_TRY(hipEventRecord(st.tl_events[4 * c + (up ? 1 : 3)], stream));
+                HIP_TRY(hipEventRecord(event_of(op.record_event), stream));
+                if (!up) st.used_buf[op.stage] = true;
+                break;
             }
-        }
-        if (trace) HIP_TRY(hipEventRecord(st.tl_events[4 * c + 3], st.d2h));
-        HIP_TRY(hipEventRecord(st.d2h_done[b], st.d2h));
-        st.used_buf[b] = true;
-        if (paced) {
-            hipLaunchKernelGGL(publish_ticket_kernel, dim3(1), dim3(1), 0, st.d2h, (uint64_t)(st.ticket_word + 1),
-                               st.seq + c + 1);
-            HIP_TRY(hipGetLastError());
+            case RT_OP_KERNEL:
+                HIP_TRY(hipStreamWaitEvent(st.comp, event_of(op.wait_event), 0));
+                rc = enqueue_kernels(plans[c], (const uint8_t*)tab.dev.ptr + plan_off[c], seed, noise_mode, d_clip_coef,
+                                     d_skip, st.comp);
+                if (rc != RT_OK) return rc;
+                HIP_TRY(hipEventRecord(event_of(op.record_event), st.comp));
+                break;
+            case RT_OP_PUBLISH:
+                hipLaunchKernelGGL(publish_ticket_kernel, dim3(1), dim3(1), 0, st.d2h, (uint64_t)(st.ticket_word + 1),
+                                   op.value);
+                HIP_TRY(hipGetLastError());
+                break;
+            case RT_OP_TICKET:
+                st.seq += chunks.size();
+                tab.ticket = st.tickets_issued + 1;
+                tab.in_flight = true;
+                // ticket: published when the last D2H of this call has landed (D2H follows compute, so
+                // device-resident arrays are final by then as well)
+                ++st.tickets_issued;
+                hipLaunchKernelGGL(publish_ticket_kernel, dim3(1), dim3(1), 0, st.d2h, (uint64_t)st.ticket_word,
+                                   st.tickets_issued);
+                HIP_TRY(hipGetLastError());
+                break;
+            default: return fail(RT_EHIP, "internal: unknown operation %u in the schedule", op.kind);
         }
     }
-    st.seq += chunks.size();
-    tab.ticket = st.tickets_issued + 1;
-    tab.in_flight = true;
-    // ticket: published when the last D2H of this call has landed (D2H follows compute, so
-    // device-resident arrays are final by then as well)
-    ++st.tickets_issued;
-    hipLaunchKernelGGL(publish_ticket_kernel, dim3(1), dim3(1), 0, st.d2h, (uint64_t)st.ticket_word,
-                       st.tickets_issued);
-    HIP_TRY(hipGetLastError());
+    (void)streams;
     if (ticket_out) *ticket_out = st.tickets_issued;
     if (trace) st.timeline.assign(4 * chunks.size(), 0.0f);
     return RT_OK;
@@ -1619,6 +1736,12 @@ static int streamed_enqueue(rt_handle* h, const rt_tensor_desc* descs, uint32_t 
         for (bool& u : st.used_buf) u = false;
         st.pending = false;
         for (auto& r : st.ring) r.in_flight = false;
+        // The failed call may have published chunk counts beyond what `seq` says (it advances only when a
+        // call succeeds): the next paced call must not take those for its own chunks coming back.
+        if (st.ticket_word) {
+            const uint64_t published = __atomic_load_n((const uint64_t*)(st.ticket_word + 1), __ATOMIC_ACQUIRE);
+            if (published > st.seq) st.seq = published;
+        }
         memcpy(g_err, saved, sizeof(saved));
     }
     return rc;

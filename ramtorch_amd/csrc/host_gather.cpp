@@ -349,6 +349,63 @@ PyObject* verify_layout(PyObject*, PyObject* const* args, Py_ssize_t nargs) {
     Py_RETURN_TRUE;
 }
 
+// dict_versions(dicts, out_addr, n) / verify_versions(dicts, expect_addr, n) -> bool
+// A recorded layout keeps the addresses of the two state tensors of every parameter and does not
+// read the state dicts again while it is in use, so nothing else may change them either.  CPython
+// stamps every dict with a version that changes whenever the dict is modified (ma_version_tag);
+// dict_versions writes the stamps of n dicts as uint64 to out_addr, verify_versions compares them:
+// a state tensor that was replaced, removed or added shows as a changed stamp, for one load per
+// dict.  (Interpreters without the stamp, 3.12 and later: dict_versions fails and no layout is recorded.)
+PyObject* dict_versions(PyObject*, PyObject* const* args, Py_ssize_t nargs) {
+#if PY_VERSION_HEX >= 0x030C0000
+    PyErr_SetString(PyExc_NotImplementedError, "this interpreter's dicts carry no version stamp");
+    return nullptr;
+#else
+    if (nargs != 3 || !PyList_CheckExact(args[0])) {
+        PyErr_SetString(PyExc_TypeError, "dict_versions(list, address, n)");
+        return nullptr;
+    }
+    auto* out = reinterpret_cast<uint64_t*>(PyLong_AsUnsignedLongLong(args[1]));
+    const Py_ssize_t n = PyLong_AsSsize_t(args[2]);
+    if (PyErr_Occurred()) return nullptr;
+    if (PyList_GET_SIZE(args[0]) != n || (n > 0 && !out)) {
+        PyErr_SetString(PyExc_ValueError, "list length and n differ");
+        return nullptr;
+    }
+    for (Py_ssize_t i = 0; i < n; ++i) {
+        PyObject* d = PyList_GET_ITEM(args[0], i);
+        if (!PyDict_Check(d)) {
+            PyErr_SetString(PyExc_TypeError, "not a dict");
+            return nullptr;
+        }
+        out[i] = reinterpret_cast<PyDictObject*>(d)->ma_version_tag;
+    }
+    Py_RETURN_NONE;
+#endif
+}
+
+PyObject* verify_versions(PyObject*, PyObject* const* args, Py_ssize_t nargs) {
+#if PY_VERSION_HEX >= 0x030C0000
+    Py_RETURN_FALSE;
+#else
+    if (nargs != 3 || !PyList_CheckExact(args[0])) {
+        PyErr_SetString(PyExc_TypeError, "verify_versions(list, address, n)");
+        return nullptr;
+    }
+    const auto* expect = reinterpret_cast<const uint64_t*>(PyLong_AsUnsignedLongLong(args[1]));
+    const Py_ssize_t n = PyLong_AsSsize_t(args[2]);
+    if (PyErr_Occurred()) return nullptr;
+    if (PyList_GET_SIZE(args[0]) != n || (n > 0 && !expect)) Py_RETURN_FALSE;
+    constexpr Py_ssize_t kAhead = 16;
+    for (Py_ssize_t i = 0; i < n; ++i) {
+        if (i + kAhead < n) touch(PyList_GET_ITEM(args[0], i + kAhead));
+        PyObject* d = PyList_GET_ITEM(args[0], i);
+        if (!PyDict_Check(d) || reinterpret_cast<PyDictObject*>(d)->ma_version_tag != expect[i]) Py_RETURN_FALSE;
+    }
+    Py_RETURN_TRUE;
+#endif
+}
+
 // set_types(torch.Tensor, torch.nn.Parameter): only objects of exactly these types take the fast path.
 PyObject* set_types(PyObject*, PyObject* args) {
     PyObject *a = nullptr, *b = nullptr;
@@ -369,6 +426,10 @@ PyMethodDef methods[] = {
      "rt_tensor_desc rows of the plain tensors of one param group"},
     {"verify_layout", reinterpret_cast<PyCFunction>(reinterpret_cast<void (*)()>(verify_layout)), METH_FASTCALL,
      "whether every parameter and gradient of a recorded layout is still where it was"},
+    {"dict_versions", reinterpret_cast<PyCFunction>(reinterpret_cast<void (*)()>(dict_versions)), METH_FASTCALL,
+     "modification stamps of a list of dicts"},
+    {"verify_versions", reinterpret_cast<PyCFunction>(reinterpret_cast<void (*)()>(verify_versions)), METH_FASTCALL,
+     "whether none of the dicts has been modified since dict_versions"},
     {"set_types", set_types, METH_VARARGS, "register torch.Tensor and torch.nn.Parameter"},
     {nullptr, nullptr, 0, nullptr},
 };

@@ -51,17 +51,22 @@ def copy_stochastic_(target: torch.Tensor, source: torch.Tensor, seed=0, *, nois
     with ``seed``; here they come from Philox4x32-10 keyed by ``seed`` (or from
     ``noise``, an int16 tensor, for reproducible tests).  With ``reference_noise`` the
     bits are drawn exactly as the reference draws them (adamw.py:10-21), which makes the
-    result bit-identical to the reference's under the same torch build.  Both tensors must
-    be contiguous GPU tensors; a CPU ``target`` is filled through a GPU temporary.
+    result bit-identical to the reference's under the same torch build.  The rounding runs on the
+    GPU: a CPU ``source`` is uploaded to the current GPU first (the reference rounds wherever
+    ``source`` lives, adamw.py:10; here the integer arithmetic is the same and only the place differs),
+    a CPU or non-contiguous ``target`` is filled through a GPU temporary.
     """
     if source.dtype != torch.float32 or target.dtype != torch.bfloat16:
         raise TypeError("copy_stochastic_ rounds float32 -> bfloat16")
     if source.numel() != target.numel():
         raise ValueError("target and source sizes differ")
     with torch.no_grad():
-        if not source.is_cuda:
-            raise RuntimeError("copy_stochastic_ needs a GPU source tensor (no CPU implementation)")
         N.lib()
+        if not torch.cuda.is_available():
+            raise RuntimeError("copy_stochastic_ needs a GPU: the rounding runs only as a HIP kernel")
+        if not source.is_cuda:
+            # the GPU of the target if it has one, else the current one
+            source = source.to(target.device if target.is_cuda else f"cuda:{torch.cuda.current_device()}")
         src = source.contiguous()
         dst = target if (target.is_cuda and target.is_contiguous()) else torch.empty(
             target.shape, dtype=torch.bfloat16, device=source.device)
@@ -103,7 +108,14 @@ class AdamW(Optimizer):
         seed: Philox key of the rounding noise.
         stream_chunk_bytes: bytes of bf16 per staged chunk of the host-resident path.
         loss_scale: gradients are divided by this inside the kernel.
-        max_grad_norm: global L2 clip computed on the GPU before the update.
+        max_grad_norm: global L2 clip computed on the GPU before the update.  A non-finite norm
+            cancels the step on the GPU (nothing is written) and the step counts it had advanced are
+            taken back when the next ``step()`` begins (``step_was_skipped()`` tells).
+        host_arrays_ordered (attribute, default False): set it when work queued on the current
+            stream may still be writing *pinned* host parameters or states when an update is handed
+            over with ``step_param`` (a ``p.data.copy_(gpu_tensor, non_blocking=True)``, a weight
+            sync): the uploads of such tensors then wait for the stream.  ``step()`` itself always
+            waits for the current stream before it uploads anything from host memory.
         noise_source: "philox" (default) draws the rounding noise inside the kernel;
             "reference" draws it the way the reference does -- three ``torch.randint``
             tensors per parameter from generators seeded ``step + 42 / 69 / 420``
@@ -147,7 +159,11 @@ class AdamW(Optimizer):
             raise ValueError(f"noise_source must be 'philox' or 'reference', got {noise_source!r}")
         self.noise_source = noise_source
         self.last_grad_norm: Optional[torch.Tensor] = None  # [norm, clip_coef, found_inf bits, -] on the GPU
+        self._skip_check = None           # per device of the last step with max_grad_norm: (event, host copy of the
+                                          # norm record, [(state, step count before)]) -- see _settle_skipped_step
+        self.last_step_skipped = False    # as of the last _settle_skipped_step()
         self.fuse_in_backward = True      # the hook of make_post_accumulate_hook() is live
+        self.host_arrays_ordered = False  # step_param: uploads from pinned host p / m / v wait for the current stream
         self.max_inflight_bytes = 2 << 30  # gradients kept alive for updates still in flight (step_param)
         self.max_inflight_calls = 2       # staging chunks handed to the copy pipeline and not finished yet
         self._poll_seconds = 0.0002       # completion is read from host memory; no runtime call while waiting
@@ -180,12 +196,13 @@ class AdamW(Optimizer):
     # to configure itself travels in one extra entry, so that copies and unpickled optimizers step.
     _CONFIG_DEFAULTS = dict(chunk_size=64, optim_state_dtype=torch.bfloat16, ema_squared_dtype=None,
                             optim_state_device="cpu", seed=0, stream_chunk_bytes=256 << 20, loss_scale=1.0,
-                            max_grad_norm=None, noise_source="philox", fuse_in_backward=True,
+                            max_grad_norm=None, noise_source="philox", fuse_in_backward=True, host_arrays_ordered=False,
                             max_inflight_bytes=2 << 30, max_inflight_calls=2, _poll_seconds=0.0002,
                             gather_min_tensors=256, state_placement="auto", state_pool_min_bytes=1 << 30,
                             assume_static_layout=False)
 
     def __getstate__(self):
+        self._settle_skipped_step()
         self._materialize_frozen_steps()
         st = dict(super().__getstate__())
         st["ramtorch_amd_config"] = {k: getattr(self, k, d) for k, d in self._CONFIG_DEFAULTS.items()}
@@ -208,8 +225,10 @@ class AdamW(Optimizer):
         self._state_lists = {}
         self._frozen = None   # steps were materialised by whoever produced `state` (__getstate__ / state_dict)
         self._freeze_requested = bool(self.__dict__.get("assume_static_layout", False))
+        self._skip_check = None
         for k, d in (("_state_pools", {}), ("state_placement_report", None), ("_gather_bufs", {}),
-                     ("_gather_stat", None), ("last_grad_norm", None), ("layout_refreezes", 0)):
+                     ("_gather_stat", None), ("last_grad_norm", None), ("layout_refreezes", 0),
+                     ("last_step_skipped", False)):
             self.__dict__.setdefault(k, d)
         for k, make in (("_stepped_early", set), ("_inflight", list), ("_early_batch", dict)):
             if k not in self.__dict__:
@@ -220,6 +239,7 @@ class AdamW(Optimizer):
         parameter index, ``param_groups``) plus one extra top-level entry with the Philox
         seed, so that a resumed run draws the noise it would have drawn.  torch's loader
         ignores entries it does not know, so the reference can read these checkpoints."""
+        self._settle_skipped_step()
         self._materialize_frozen_steps()
         sd = super().state_dict()
         sd["ramtorch_amd"] = {"seed": self.seed}
@@ -258,6 +278,38 @@ class AdamW(Optimizer):
         self._recs = None
         self._desc_cache = {}
         self._state_lists = {}
+
+    # -- a step that the skip flag cancelled must not have counted -------------------------------------
+    def _settle_skipped_step(self) -> bool:
+        """With ``max_grad_norm``, a non-finite global gradient norm makes the kernels leave everything
+        untouched (the GPU decides; the host does not wait for it).  ``state["step"]`` has been advanced
+        by then, as adamw.py:177 advances it before the arithmetic -- but a step that did not happen
+        must not count: bias corrections and the Philox counter would run one ahead of the data for
+        the rest of training (torch's GradScaler never calls ``step()`` on such gradients).  So the
+        norm record of a step is copied to pinned host memory behind its kernels, and the next
+        ``step()`` (or ``state_dict()``, pickling, ``step_was_skipped()``) reads it -- it landed
+        long ago, nothing stalls -- and takes the increments back if the step was cancelled.
+        Returns whether it was."""
+        checks = self.__dict__.get("_skip_check")
+        if not checks:
+            return False
+        self._skip_check = None
+        skipped = False
+        for event, host, journal in checks:
+            event.synchronize()
+            if int(host.view(torch.int32)[2]) != 0:
+                skipped = True
+                for state, old in reversed(journal):
+                    state["step"] = old
+        self.last_step_skipped = skipped
+        return skipped
+
+    def step_was_skipped(self) -> bool:
+        """Whether the most recent ``step()`` was cancelled by a non-finite gradient norm (waits for
+        that step's norm pass if it has not finished yet)."""
+        if self.__dict__.get("_skip_check"):
+            self._settle_skipped_step()
+        return self.last_step_skipped
 
     # -- state ---------------------------------------------------------------------
     def _state_dtype(self, key: str) -> torch.dtype:
@@ -407,6 +459,7 @@ class AdamW(Optimizer):
         if not torch.cuda.is_available():
             raise RuntimeError("ramtorch_amd.AdamW.step needs a GPU: the update runs only as HIP kernels")
 
+        self._settle_skipped_step()
         if (self._frozen is not None and noise is None and debug_out is None and grads is None
                 and not self._stepped_early and not self._early_batch and not self._inflight):
             if self._step_frozen():
@@ -458,6 +511,8 @@ class AdamW(Optimizer):
             gather = G.module()
         gathered: Dict[int, list] = {}    # dev -> [descriptor buffer, rows used]
         cen_jobs: Dict[int, list] = {}    # dev -> [(entry, rows, row_len)] of gradients to centralize
+        counted: Dict[int, list] = {}     # dev -> [(state, step count before)] of the tensors under max_grad_norm
+        skip_checks = []
 
         for gi, group in enumerate(self.param_groups):
             beta1, beta2 = group["betas"]
@@ -503,6 +558,8 @@ class AdamW(Optimizer):
                     state = r.state
                 step = state["step"] + 1  # adamw.py:177
                 journal.append((state, state["step"]))
+                if self.max_grad_norm is not None:
+                    counted.setdefault(r.dev, []).append(journal[-1])
                 state["step"] = step
                 if step != last_step:
                     key = (gi, step, lr, beta1, beta2, eps, wd, cen)
@@ -599,6 +656,12 @@ class AdamW(Optimizer):
                     out = F.grad_norm(h, gl, inv_loss_scale=inv_loss_scale, max_norm=self.max_grad_norm)
                     self.last_grad_norm = out
                     clip, skip = out[1:2], out[2:3]
+                    # the record goes to pinned host memory behind the norm pass; the next step reads it there
+                    host = torch.empty(4, dtype=torch.float32, pin_memory=True)
+                    host.copy_(out, non_blocking=True)
+                    event = torch.cuda.Event()
+                    event.record()
+                    skip_checks.append((event, host, counted.get(dev, [])))
                 launched[0] = True
                 if descs is not None:
                     F.launch_resident(h, descs, scalars, seed=self.seed, explicit_noise=explicit, clip_coef=clip,
@@ -609,6 +672,8 @@ class AdamW(Optimizer):
                                     chunk_elems=chunk_elems, clip_coef=clip, skip=skip, descs=stm_descs)
         for dst, tmp in writeback:
             dst.copy_(tmp)
+        if skip_checks:
+            self._skip_check = skip_checks
         if self._freeze_requested:
             self._record_layout(gathered, plain, resident, streamed, scalar_key, explicit)
 
@@ -628,8 +693,12 @@ class AdamW(Optimizer):
 
         What ends a recorded layout: ``add_param_group``, ``load_state_dict``, ``unfreeze_layout()``,
         and any step whose check fails (a gradient appeared, vanished, moved or changed dtype; a
-        parameter moved; a ``params`` list changed) -- that step runs the full path, with the same
-        results, and records the layout again if ``assume_static_layout`` is set.  While a layout is
+        parameter moved; a ``params`` list changed; an entry of ``optimizer.state`` or of a
+        parameter's state dict was assigned, added or removed) -- that step runs the full path, with
+        the same results, and records the layout again if ``assume_static_layout`` is set.  Not
+        seen: the storage of a state tensor exchanged in place (``state["ema"].data = ...``,
+        ``set_``); the recorded storages are kept alive, so such a step still updates the memory that
+        was recorded.  While a layout is
         recorded, ``state[p]["step"]`` of the recorded tensors lags behind; it is brought up to date
         by ``state_dict()``, ``unfreeze_layout()`` and by any step that takes the full path."""
         self._freeze_requested = True
@@ -651,7 +720,12 @@ class AdamW(Optimizer):
         k = fz["pending"]
         for st in fz["states"]:
             st["step"] += k
+        # the recorded step counts move along, so that the next recorded step builds its scalars
+        # for the step it really is (the descriptors' own step words have advanced all the while)
+        fz["keys"] = [(gi, st + k) for gi, st in fz["keys"]]
         fz["pending"] = 0
+        # these writes are the optimizer's own: the state dicts' modification stamps are taken again
+        G.module().dict_versions(fz["state_dicts"], fz["versions"].ctypes.data, len(fz["state_dicts"]))
 
     def _record_layout(self, gathered, plain, resident, streamed, scalar_key, explicit) -> None:
         self._frozen = None
@@ -683,8 +757,21 @@ class AdamW(Optimizer):
             keys[idx] = (gi, st)
         if any(x is None for x in keys):
             return
+        # The descriptors keep the addresses of the state tensors.  Their storages are held, so that the
+        # addresses stay valid whatever happens to the tensors, and every state dict's modification
+        # stamp is noted (with that of ``self.state`` itself): a state that is replaced, removed or
+        # added shows there, one load per dict and step.
+        states = [self.state[params[i]] for i in ids]
+        state_dicts = states + [self.state]
+        versions = np.zeros(len(state_dicts), np.uint64)
+        try:
+            G.module().dict_versions(state_dicts, versions.ctypes.data, len(state_dicts))
+        except (NotImplementedError, AttributeError):
+            return    # no stamps in this interpreter (or an older helper): no recorded layouts
+        keep = [t.untyped_storage() for st in states for t in (st["ema"], st["ema_squared"])]
         self._frozen = {"dev": dev, "descs": descs, "params": params, "expect": expect,
-                        "states": [self.state[params[i]] for i in ids], "keys": keys, "pending": 0,
+                        "states": states, "state_dicts": state_dicts, "versions": versions, "keep": keep,
+                        "keys": keys, "pending": 0,
                         "group_lists": [(g["params"], len(g["params"])) for g in self.param_groups]}
         if not self.assume_static_layout:
             self._freeze_requested = False
@@ -698,7 +785,9 @@ class AdamW(Optimizer):
             for g, (lst, n) in zip(groups, fz["group_lists"]))
         ok = ok and self.max_grad_norm is None and getattr(self, "noise_source", "philox") == "philox"
         if ok:
-            ok = G.module().verify_layout(fz["params"], fz["expect"].ctypes.data, len(fz["params"]))
+            ok = (fz["state_dicts"][-1] is self.state
+                  and G.module().verify_versions(fz["state_dicts"], fz["versions"].ctypes.data, len(fz["state_dicts"]))
+                  and G.module().verify_layout(fz["params"], fz["expect"].ctypes.data, len(fz["params"])))
         if not ok:
             self.layout_refreezes += 1
             self.unfreeze_layout()
@@ -823,27 +912,51 @@ class AdamW(Optimizer):
                 g = g.contiguous()
             if g.dtype not in (torch.bfloat16, torch.float32, torch.float16):
                 g = g.to(torch.float32)
-            step = state["step"] + 1
-            state["step"] = step
+            old_step = state["step"]
+            step = old_step + 1    # adamw.py:177; written to the state only when nothing can raise any more
             inv_loss_scale = 1.0 / self.loss_scale if self.loss_scale != 1.0 else 1.0
             cen = group["centralization"]
             sc = [F.make_scalars(group["lr"], tuple(group["betas"]), group["eps"], group["weight_decay"], step,
                                  centralization=cen, inv_loss_scale=inv_loss_scale)]
-            e = F.Entry(p=p.data, g=g, m=r.m, v=r.v, step=step, scalars_idx=0, tensor_id=r.tensor_id)
+            e = F.Entry(p=p.data, g=g, m=r.m, v=r.v, step=step, scalars_idx=0, tensor_id=r.tensor_id,
+                        ordered=bool(self.__dict__.get("host_arrays_ordered", False)))
+            for t, what in ((e.p, "param"), (e.g, "grad"), (e.m, "state"), (e.v, "state")):
+                F.dtype_code(t.dtype, what)     # an unsupported dtype raises here
+            if g.numel() != p.numel():
+                raise ValueError("step_param: the gradient's size differs from the parameter's")
             if cen != 0:
                 e.row_mean, e.row_len = self._row_means(g, dev, inv_loss_scale)
             h = _handle(dev)
-            with torch.cuda.device(dev):
-                if e.p.is_cuda and e.m.is_cuda and e.v.is_cuda:
-                    F.step_resident(h, [e], sc, seed=self.seed, explicit_noise=False)  # stream-ordered already
-                else:
-                    # Tensors are handed to the copy pipeline in pieces of exactly one staging chunk
-                    # (a tensor may be cut, at a multiple of 8 elements): chunks of equal size keep
-                    # H2D and D2H overlapped, a run of unequal tensors would not.
-                    batch = self._early_batch.setdefault(dev, [[], 0])
-                    batch[0].append([e, sc[0], 0])      # entry, its scalars, elements already handed over
-                    batch[1] += e.p.numel()
-                    self._flush_early_batch(dev, final=False)
+            state["step"] = step
+            handed_over = False    # part of this tensor is already on the copy pipeline: the step counts
+            try:
+                with torch.cuda.device(dev):
+                    if e.p.is_cuda and e.m.is_cuda and e.v.is_cuda:
+                        F.step_resident(h, [e], sc, seed=self.seed, explicit_noise=False)  # stream-ordered already
+                    else:
+                        # Tensors are handed to the copy pipeline in pieces of exactly one staging chunk
+                        # (a tensor may be cut, at a multiple of 8 elements): chunks of equal size keep
+                        # H2D and D2H overlapped, a run of unequal tensors would not.
+                        batch = self._early_batch.setdefault(dev, [[], 0])
+                        batch[0].append([e, sc[0], 0])      # entry, its scalars, elements already handed over
+                        batch[1] += e.p.numel()
+                        try:
+                            self._flush_early_batch(dev, final=False)
+                        except BaseException:
+                            # nothing of this tensor has been handed over unless a piece of it was: take it
+                            # out of the batch again when it is still whole
+                            if batch[0] and batch[0][-1][0] is e and batch[0][-1][2] == 0:
+                                batch[0].pop()
+                                batch[1] -= e.p.numel()
+                                if not batch[0]:
+                                    self._early_batch.pop(dev, None)
+                            else:
+                                handed_over = True
+                            raise
+            except BaseException:
+                if not handed_over:
+                    state["step"] = old_step
+                raise
         self._stepped_early.add(id(p))
 
     def _flush_early_batch(self, dev: int, final: bool) -> None:

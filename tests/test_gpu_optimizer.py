@@ -433,6 +433,89 @@ def test_clip_with_centralization():
     h.close()
 
 
+def test_copy_stochastic_with_a_cpu_source():
+    """adamw.py:6-30 rounds wherever ``source`` lives; here a CPU source goes through the GPU.  Same bits as
+    the integer closed form, into a CPU target and into a GPU target, with Philox and with explicit noise."""
+    n = 70_001
+    src = torch.randn(n) * 0.02
+    noise = torch.randint(-32768, 32768, (n,), dtype=torch.int16)
+    for tgt in (torch.empty(n, dtype=torch.bfloat16), torch.empty(n, dtype=torch.bfloat16, device="cuda")):
+        ramtorch_amd.copy_stochastic_(tgt, src, seed=5)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(bits16(tgt), oracle.sr_copy(src.numpy(), seed=5))
+        ramtorch_amd.copy_stochastic_(tgt, src, noise=noise)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(bits16(tgt), oracle.sr_copy(src.numpy(), noise=noise.numpy()))
+    # 2-d, a non-contiguous CPU target
+    src2 = (torch.randn(60, 50) * 0.02)
+    tgt2 = torch.empty(50, 60, dtype=torch.bfloat16).t()
+    ramtorch_amd.copy_stochastic_(tgt2, src2, seed=6)
+    np.testing.assert_array_equal(bits16(tgt2.contiguous()), oracle.sr_copy(src2.numpy().ravel(), seed=6))
+
+
+@pytest.mark.parametrize("storage", ["cuda", "cpu"])
+def test_a_step_cancelled_by_a_non_finite_norm_does_not_count(storage):
+    """max_grad_norm with an infinite gradient: the kernels leave everything as it is, and the step counts
+    the call had advanced are taken back, so that the next step is the one after the last that happened --
+    same bias corrections, same Philox counter word (the reference increments right before its arithmetic,
+    adamw.py:177; torch's GradScaler does not call step() at all on such gradients)."""
+    shapes = [(256, 64), (3 * 8192 + 11,)]
+    ps, grads = _make_params(shapes, 720, device=storage if storage == "cuda" else "cpu")
+    if storage == "cpu":
+        ps = [torch.nn.Parameter(p.detach().pin_memory()) for p in ps]
+    opt = ramtorch_amd.AdamW(ps, storage_device=storage, seed=21, max_grad_norm=1e9, **HP0)
+    gmap = {p: g.clone() for p, g in zip(ps, grads)}
+    sc = lambda step: oracle.scalars_from_hparams(step=step, apply_clip=True, **HP0)
+    model = [(bits16(p), np.zeros(p.numel(), np.uint16), np.zeros(p.numel(), np.uint16)) for p in ps]
+
+    def good_step(step):
+        opt.step(grads=gmap)
+        torch.cuda.synchronize()
+        for i, (p, (po, mo, vo)) in enumerate(zip(ps, model)):
+            oracle.step_tensor(po, bits16(gmap[p]), mo, vo, sc(step), clip_coef=np.float32(1.0), seed=21, step=step, tensor_id=i)
+            np.testing.assert_array_equal(bits16(p), po, err_msg=f"step {step} param {i}")
+            np.testing.assert_array_equal(bits16(opt.state[p]["ema"]), mo, err_msg=f"step {step} ema {i}")
+            np.testing.assert_array_equal(bits16(opt.state[p]["ema_squared"]), vo, err_msg=f"step {step} ema_squared {i}")
+
+    good_step(1)
+    assert not opt.step_was_skipped()
+    keep = gmap[ps[1]][5].clone()
+    gmap[ps[1]][5] = float("inf")
+    opt.step(grads=gmap)                       # cancelled on the GPU
+    torch.cuda.synchronize()
+    for p, (po, mo, vo) in zip(ps, model):
+        np.testing.assert_array_equal(bits16(p), po)
+        np.testing.assert_array_equal(bits16(opt.state[p]["ema"]), mo)
+    assert opt.step_was_skipped()
+    assert [opt.state[p]["step"] for p in ps] == [1, 1]
+    assert [v["step"] for v in opt.state_dict()["state"].values()] == [1, 1]
+    gmap[ps[1]][5] = keep
+    good_step(2)                               # the step after step 1, bit for bit
+    assert not opt.step_was_skipped() and [opt.state[p]["step"] for p in ps] == [2, 2]
+    # cancelled again, and this time the next step() itself finds out
+    gmap[ps[0]][0, 0] = float("nan")
+    opt.step(grads=gmap)
+    gmap[ps[0]][0, 0] = 0.0
+    good_step(3)
+
+
+def test_step_param_that_raises_leaves_the_step_count_alone():
+    ps, grads = _make_params([(64, 32)], 730)
+    opt = ramtorch_amd.AdamW(ps, storage_device="cuda", seed=2, **HP0)
+    opt.step_param(ps[0], grads[0])
+    opt.step()
+    assert opt.state[ps[0]]["step"] == 1
+    before = bits16(ps[0])
+    with pytest.raises(ValueError):
+        opt.step_param(ps[0], grads[0].view(-1)[:100])           # a gradient of the wrong size
+    torch.cuda.synchronize()
+    assert opt.state[ps[0]]["step"] == 1 and id(ps[0]) not in opt._stepped_early
+    np.testing.assert_array_equal(bits16(ps[0]), before)
+    opt.step_param(ps[0], grads[0])                             # and the parameter can still be stepped
+    opt.step()
+    assert opt.state[ps[0]]["step"] == 2
+
+
 def test_copy_stochastic():
     n = 100_003
     src = torch.randn(n, device="cuda") * 0.02
@@ -815,6 +898,22 @@ def test_frozen_layout_steps_like_the_full_path_and_notices_moved_gradients():
         assert a._frozen is not None and a._frozen["pending"] == k + 1 and a.layout_refreezes == 0
     sd_a, sd_b = a.state_dict(), b.state_dict()       # brings the lagging step counts up to date
     assert [sd_a["state"][i]["step"] for i in sorted(sd_a["state"])] == [sd_b["state"][i]["step"] for i in sorted(sd_b["state"])]
+    # ... and the recorded layout stays in use afterwards, with the scalars of the step it really is
+    # (bias corrections and step size come from the step count: one taken from before the save would
+    # show in every element)
+    a.step(); b.step(); same()
+    assert a._frozen is not None and a._frozen["pending"] == 1 and a.layout_refreezes == 0
+    twin = copy.deepcopy(a)                           # pickling brings the counts up to date as well
+    assert [twin.state[p]["step"] for g in twin.param_groups for p in g["params"]] == [b.state[p]["step"] for p in ps_b]
+    del twin
+    a.step(); b.step(); same()
+    assert a._frozen is not None and a._frozen["pending"] == 1 and a.layout_refreezes == 0
+    # a state tensor replaced behind the optimizer's back: noticed, full path, same bits as doing it to b
+    for opt, ps in ((a, ps_a), (b, ps_b)):
+        opt.state[ps[3]]["ema"] = opt.state[ps[3]]["ema"].clone()
+    a.step(); b.step(); same()
+    assert a.layout_refreezes == 1 and a._frozen is not None
+    a.layout_refreezes = 0
     # a gradient moves: caught, the step takes the full path and records the layout again
     for ps in (ps_a, ps_b):
         ps[7].grad = ps[7].grad.clone()

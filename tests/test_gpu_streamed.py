@@ -100,7 +100,8 @@ def test_unpinned_gradients_go_up_through_bounce_buffers(handle, chunk_elems):
     """The reference's offload flow leaves the gradients in ordinary CPU memory (linear.py:416-427):
     host threads copy them into pinned bounce buffers chunk by chunk.  More chunks than bounce
     buffers, pinned and unpinned gradients in one call, two calls in a row (the buffer index
-    runs on across calls), and an unpinned parameter next to pinned states."""
+    runs on across calls), and an unpinned parameter next to pinned states (it goes up through the
+    upload slots and its update comes back through the download slots)."""
     lens = [30_011, 8, 0, 4096, 100_000, 5, 8193]
     before = handle.streamed_bounce_stats()
     state = []
@@ -116,7 +117,7 @@ def test_unpinned_gradients_go_up_through_bounce_buffers(handle, chunk_elems):
             G = host16(g, pin=not unpinned)
             assert G.is_pinned() != unpinned or len(g) == 0
             entries.append(F.Entry(p=P, g=G, m=M, v=V, step=step, scalars_idx=0, tensor_id=i))
-            expect_bytes += 2 * len(g) * unpinned + 2 * len(p) * (i == 4)
+            expect_bytes += 2 * len(g) * unpinned + 2 * 2 * len(p) * (i == 4)   # the unpinned parameter goes up and comes down
         F.step_streamed(handle, entries, [sc], seed=31, explicit_noise=False, chunk_elems=chunk_elems)
         for i, (p, g, m, v, P, M, V) in enumerate(state):
             oracle.step_tensor(p, g, m, v, sco, seed=31, step=step, tensor_id=i)

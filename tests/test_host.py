@@ -466,3 +466,255 @@ int main() {
     subprocess.check_call(["g++", "-std=c++17", "-O1", "-Wall", "-Werror", "-pthread", "-fsanitize=thread",
                            "-I", os.path.join(ROOT, "ramtorch_amd", "csrc"), str(src), "-o", str(exe)])
     assert subprocess.check_output([str(exe)], text=True).strip() == "ok"
+
+
+# ---- the streamed pipeline's order of operations, replayed on the CPU ---------------------------------
+# rt_streamed_schedule hands out the very list of operations the library executes for a streamed call
+# (three streams, two staging buffers per array, four bounce slots each way, events, host waits).  The
+# replay below runs such lists as the hardware may: the host issues operations in order and blocks where
+# the list says it waits; every stream runs its operations in order, each starting no earlier than the
+# event it waits for; host copies run beside all of that; which of the possible next things happens is
+# drawn at random.  Two things are checked at every start of an operation: nothing else that is running
+# touches a buffer it writes (or writes one it reads), and every buffer it reads holds what it is
+# supposed to hold.  The reference keeps its transfers apart with ping-pong buffers and events
+# (ramtorch/modules/linear.py:163-197, 267-308) and device-wide syncs (adamw.py:227-232).
+class _Replay:
+    def __init__(self, calls, rng):
+        """calls: [(ops, seq0)] executed back to back on one handle."""
+        self.rng = rng
+        self.calls = calls
+        self.violations = []
+        self.content = {}            # buffer -> tag of what it holds
+        self.running = []            # [name, reads, writes, on_finish]
+        self.queues = {s: [] for s in ("h2d", "comp", "d2h")}   # issued, not yet started: (op, awaited record or None, abs chunk)
+        self.stream_busy = {s: None for s in self.queues}
+        self.records = {}            # event id -> index of its most recent record among the issued ones
+        self.record_done = set()     # (event id, index) of completed records
+        self.record_count = {}
+        self.back = 0                # the published chunk counter
+        self.copies = {}             # ("fill" | "drain", abs chunk) -> running entry or "done"
+        speeds = [0.02, 1.0, 50.0]
+        self.weight = {k: speeds[rng.integers(3)] for k in ("host", "start", "finish", "copy")}
+        self.stream_weight = {s: speeds[rng.integers(3)] for s in ("h2d", "comp", "d2h")}
+        self._copy_weight = {}
+
+    def copy_weight(self, key):
+        if key not in self._copy_weight:     # every host copy has a speed of its own
+            self._copy_weight[key] = [0.02, 1.0, 50.0][self.rng.integers(3)]
+        return self._copy_weight[key]
+
+    def _conflict(self, name, reads, writes):
+        for other, oreads, owrites, *_ in self.running:
+            for b in writes:
+                if b in oreads or b in owrites:
+                    self.violations.append(f"{name} writes {b} while {other} uses it")
+            for b in reads:
+                if b in owrites:
+                    self.violations.append(f"{name} reads {b} while {other} writes it")
+
+    def _expect(self, name, buf, tag):
+        if self.content.get(buf) != tag:
+            self.violations.append(f"{name} finds {self.content.get(buf)} in {buf}, not {tag}")
+
+    def _start(self, name, reads, writes, expects, results):
+        self._conflict(name, reads, writes)
+        for buf, tag in expects:
+            self._expect(name, buf, tag)
+        for buf in writes:
+            self.content[buf] = ("being written by", name)
+        entry = [name, set(reads), set(writes), results]
+        self.running.append(entry)
+        return entry
+
+    def _finish(self, entry):
+        self.running.remove(entry)
+        for buf, tag in entry[3]:
+            self.content[buf] = tag
+
+    def run(self, paced_up, paced_down):
+        K = N
+        stream_of = {K.RT_OP_H2D: "h2d", K.RT_OP_KERNEL: "comp", K.RT_OP_D2H: "d2h", K.RT_OP_PUBLISH: "d2h", K.RT_OP_TICKET: "d2h"}
+        flat = [(op, seq0) for ops, seq0 in self.calls for op in ops]
+        pc = 0
+        steps = 0
+        while True:
+            steps += 1
+            assert steps < 200000, "the replay does not end"
+            actions = []
+            # -- the host: issue the next operation, unless it has to wait
+            if pc < len(flat):
+                op, seq0 = flat[pc]
+                c = seq0 + op.chunk
+                if op.kind == K.RT_OP_HOST_WAIT_BACK:
+                    if self.back >= op.value:
+                        actions.append(("host", None))
+                elif op.kind == K.RT_OP_HOST_WAIT_FILL:
+                    if self.copies.get(("fill", c), "done") == "done":
+                        actions.append(("host", None))
+                elif op.kind == K.RT_OP_HOST_WAIT_DRAIN:
+                    if self.copies.get(("drain", c), "done") == "done":
+                        actions.append(("host", None))
+                elif op.kind == K.RT_OP_HOST_WAIT_IDLE:
+                    if not any(self.queues.values()) and not any(self.stream_busy.values()):
+                        actions.append(("host", None))
+                else:
+                    actions.append(("host", None))
+            # -- streams: start the head operation when its event has fired; finish what runs
+            for s, q in self.queues.items():
+                if self.stream_busy[s] is not None:
+                    actions.append(("finish", s))
+                elif q:
+                    op, awaited, c = q[0]
+                    if awaited is None or awaited in self.record_done:
+                        actions.append(("start", s))
+            for key, entry in self.copies.items():
+                if entry != "done":
+                    actions.append(("copy", key))
+            if not actions:
+                assert pc >= len(flat) and not any(self.queues.values()), "the replay is stuck: a wait that nothing satisfies"
+                return self.violations
+            # Which of them happens: drawn with weights that differ from replay to replay by orders of
+            # magnitude (a host far ahead of the device, copies that crawl, a stream that stalls ...)
+            w = np.array([self.weight[a[0]] * (self.copy_weight(a[1]) if a[0] == "copy" else self.stream_weight.get(a[1], 1.0))
+                          for a in actions])
+            kind, arg = actions[self.rng.choice(len(actions), p=w / w.sum())]
+            if kind == "host":
+                op, seq0 = flat[pc]
+                pc += 1
+                if pc == len(flat):    # the call returns to its caller: host memory must be final
+                    for key, entry in self.copies.items():
+                        if entry != "done":
+                            self.violations.append(f"the call returns while {key} is still copying")
+                c = seq0 + op.chunk
+                if op.kind == K.RT_OP_HOST_FILL:
+                    e = self._start(f"fill({c})", [("user", c)], [("up", op.bounce)], [], [(("up", op.bounce), ("chunk", c))])
+                    self.copies[("fill", c)] = e
+                elif op.kind == K.RT_OP_HOST_DRAIN:
+                    e = self._start(f"drain({c})", [("down", op.bounce)], [("user", c)], [(("down", op.bounce), ("result", c))],
+                                    [(("user", c), ("result", c))])
+                    self.copies[("drain", c)] = e
+                elif op.kind in stream_of:
+                    awaited = None
+                    if op.wait_event != K.RT_SCHED_NONE and op.wait_event in self.records:
+                        awaited = (op.wait_event, self.records[op.wait_event])
+                    if op.record_event != K.RT_SCHED_NONE:
+                        k = self.record_count.get(op.record_event, 0)
+                        self.record_count[op.record_event] = k + 1
+                        self.records[op.record_event] = k
+                        op_record = (op.record_event, k)
+                    else:
+                        op_record = None
+                    self.queues[stream_of[op.kind]].append(((op, op_record), awaited, c))
+            elif kind == "start":
+                (op, op_record), _, c = self.queues[arg].pop(0)
+                stage = ("stage", op.stage)
+                if op.kind == K.RT_OP_H2D:
+                    src = ("up", op.bounce) if op.bounce != K.RT_SCHED_NONE else ("user", c)
+                    expects = [(src, ("chunk", c))] if op.bounce != K.RT_SCHED_NONE else []
+                    e = self._start(f"h2d({c})", [src], [stage], expects, [(stage, ("chunk", c))])
+                elif op.kind == K.RT_OP_KERNEL:
+                    e = self._start(f"kernel({c})", [stage], [stage], [(stage, ("chunk", c))], [(stage, ("result", c))])
+                elif op.kind == K.RT_OP_D2H:
+                    dst = ("down", op.bounce) if op.bounce != K.RT_SCHED_NONE else ("user", c)
+                    e = self._start(f"d2h({c})", [stage], [dst], [(stage, ("result", c))], [(dst, ("result", c))])
+                else:
+                    e = self._start("publish", [], [], [], [])
+                    e.append(op)
+                self.stream_busy[arg] = (e, op_record)
+            elif kind == "finish":
+                e, op_record = self.stream_busy[arg]
+                self.stream_busy[arg] = None
+                self._finish(e)
+                if op_record is not None:
+                    self.record_done.add(op_record)
+                if len(e) > 4 and e[4].kind == K.RT_OP_PUBLISH:
+                    self.back = max(self.back, e[4].value)
+            else:
+                e = self.copies[arg]
+                self._finish(e)
+                self.copies[arg] = "done"
+
+
+def _two_calls(n1, n2, paced_up, paced_down, batch=3):
+    """Two streamed calls on one handle, the second chained behind the first as the library chains them."""
+    a = N.streamed_schedule(n1, 0, 0, paced_up, paced_down, batch)
+    used = (1 if n1 >= 1 else 0) | (2 if n1 >= 2 else 0)     # staging buffers 0 and 1 hold chunks of the first call
+    b = N.streamed_schedule(n2, n1, used, paced_up, paced_down, batch)
+    return [(a, 0), (b, n1)]
+
+
+@pytest.mark.parametrize("paced_up,paced_down", [(False, False), (True, False), (True, True), (False, True)])
+def test_streamed_schedule_keeps_buffers_apart_under_any_interleaving(paced_up, paced_down):
+    for n1, n2 in ((1, 1), (2, 3), (5, 4), (9, 7)):
+        calls = _two_calls(n1, n2, paced_up, paced_down)
+        for seed in range(60):
+            bad = _Replay(calls, np.random.default_rng(seed)).run(paced_up, paced_down)
+            assert not bad, (n1, n2, seed, bad[:3])
+        # every chunk went through all three stages exactly once, in chunk order on every stream
+        for ops, _ in calls:
+            for kind in (N.RT_OP_H2D, N.RT_OP_KERNEL, N.RT_OP_D2H):
+                assert [o.chunk for o in ops if o.kind == kind] == list(range(len([o for o in ops if o.kind == N.RT_OP_H2D])))
+            assert [o.kind for o in ops].count(N.RT_OP_TICKET) == 1
+
+
+def _without(ops, index):
+    """The schedule with one wait taken out: a stream operation loses its event, a host wait disappears."""
+    out = []
+    for i, o in enumerate(ops):
+        if i != index:
+            out.append(o)
+        elif o.kind in (N.RT_OP_H2D, N.RT_OP_KERNEL, N.RT_OP_D2H):
+            c = N.RtSchedOp.from_buffer_copy(o)
+            c.wait_event = N.RT_SCHED_NONE
+            out.append(c)
+    return out
+
+
+@pytest.mark.parametrize("paced_up,paced_down", [(False, False), (True, True)])
+def test_streamed_schedule_replay_notices_a_missing_wait(paced_up, paced_down):
+    """The check has teeth: take any single wait that protects a buffer out of the list and some interleaving
+    shows the damage.  (The waits of a long unpaced call between its batches of chunks only keep the
+    streams' queues short; nothing is unsafe without them, and they are left out here.)"""
+    ops = N.streamed_schedule(8, 0, 0, paced_up, paced_down, 64)
+    # (paced, an upload's wait for its staging buffer is implied by the host's own wait for that chunk to
+    # have come back, two chunks earlier; it stays in the list because asynchronous calls chain on it)
+    evented = (N.RT_OP_KERNEL, N.RT_OP_D2H) if (paced_up or paced_down) else (N.RT_OP_H2D, N.RT_OP_KERNEL, N.RT_OP_D2H)
+    waits = [i for i, o in enumerate(ops)
+             if (o.kind in evented and o.wait_event != N.RT_SCHED_NONE)
+             or o.kind in (N.RT_OP_HOST_WAIT_BACK, N.RT_OP_HOST_WAIT_FILL, N.RT_OP_HOST_WAIT_DRAIN)]   # (a single call: nothing before it to wait for)
+    assert len(waits) >= 20
+    for i in waits:
+        broken = _without(ops, i)
+        caught = False
+        for seed in range(300):
+            try:
+                bad = _Replay([(broken, 0)], np.random.default_rng(seed)).run(paced_up, paced_down)
+            except AssertionError:     # a replay that cannot end is a broken schedule too
+                bad = ["stuck"]
+            if bad:
+                caught = True
+                break
+        assert caught, (i, ops[i].kind, ops[i].chunk)
+
+
+def test_recorded_layout_keeps_its_step_counts_in_step_with_the_states():
+    """Bringing the lagging step counts of a recorded layout up to date (state_dict(), pickling) must move
+    the recorded counts along: the next recorded step builds its bias corrections from them."""
+    from ramtorch_amd import _gather as G
+    if G.module() is None:
+        pytest.skip("the gather helper is not built")
+    p = torch.nn.Parameter(torch.zeros(8, dtype=torch.bfloat16))
+    opt = ramtorch_amd.AdamW([p], storage_device="cpu")
+    st = opt.state[p]
+    st["step"] = 2
+    dicts = [st, opt.state]
+    versions = np.zeros(2, np.uint64)
+    G.module().dict_versions(dicts, versions.ctypes.data, 2)
+    opt._frozen = {"pending": 3, "states": [st], "keys": [(0, 2)], "state_dicts": dicts, "versions": versions}
+    opt._materialize_frozen_steps()
+    assert st["step"] == 5 and opt._frozen["keys"] == [(0, 5)] and opt._frozen["pending"] == 0
+    # the optimizer's own writes do not count as somebody else's: the stamps were taken again
+    assert G.module().verify_versions(dicts, versions.ctypes.data, 2)
+    st["ema"] = st["ema"].clone()            # somebody else's does
+    assert not G.module().verify_versions(dicts, versions.ctypes.data, 2)
+    opt._frozen = None

@@ -114,3 +114,30 @@ def test_static_grad_norm_matches_the_allocating_entry_point_twice_in_a_row():
     finally:
         torch.cuda.synchronize()
         h.close()
+
+
+def test_static_grad_norm_calls_from_two_handles_and_streams_take_turns():
+    """Two handles, each on a stream of its own, call the static entry point back to back without any
+    synchronisation in between: both use the GPU's one array, and each call waits on the GPU for the one
+    before it, so every result is the one the allocating entry point gives."""
+    h1, h2 = N.Handle(0), N.Handle(0)
+    try:
+        s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+        sets = [_make_grads([200_000 + 8192 * k, 1 << 20, 77], 20 + k) for k in range(6)]
+        want = []
+        for g in sets:
+            a, _ = _both(h1, g, max_norm=0.25)
+            want.append(a)
+        outs = [torch.full((4,), float("nan"), device="cuda") for _ in sets]
+        ds = [_descs(g) for g in sets]
+        torch.cuda.synchronize()
+        for k, (d, out) in enumerate(zip(ds, outs)):
+            h, s = ((h1, s1), (h2, s2))[k % 2]
+            h.grad_norm_static(F._descs_ptr(d), len(d), 1.0, 0.25, out.data_ptr(), s.cuda_stream)
+        torch.cuda.synchronize()
+        for k, (out, a) in enumerate(zip(outs, want)):
+            assert (out.cpu().numpy().view(np.uint32)[:3] == a).all(), k
+    finally:
+        torch.cuda.synchronize()
+        h1.close()
+        h2.close()
