@@ -37,6 +37,13 @@ ema~N(0,1e-4), ema_squared=N(0,1e-3)^2, stored bf16):
             backward pass would hand its gradient over (last tensor first), and
             step() only waits: the grad hand-off from ramtorch.Linear's
             post-accumulate hook
+  any       one transformer layer of the set (9 tensors, 218 112 000 elements) with bf16 parameters
+            and gradients and both states in fp64 (the reference upcasts any dtype, adamw.py:160-170,
+            and writes what is not bf16 back with a plain copy_): the runtime-typed kernel that
+            serves the layouts without a templated instance; 34 bytes per element
+  pageable  a 16 GB prefix of the set with parameters and states in ordinary (not pinned) CPU memory,
+            the third kind of input adamw.py:152-170 accepts: up through the library's pinned
+            bounce buffers, filled by host threads, and down through them again
   offload_ref  the same set as the reference's own offload flow leaves it
             (linear.py:416-427 -> adamw.py:167): pinned CPU params and states
             and the gradients on the CPU too (in the pinned memory that
@@ -73,10 +80,11 @@ OFFLINE_TRAFFIC = {
 }
 HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
 METRIC = "SR-AdamW step: params/sec + achieved HBM GB/s (% of peak), 8B bf16 set, 1 GPU"
-RESIDENT = ("llama8b", "cfg0", "small", "mixed", "central")
-HOST = ("streamed", "hooked", "offload_ref")
-UPDATE_BYTES = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 20, "central": 14}   # per element, update launch only
-STEP_BYTES = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 24, "central": 16, "streamed": 12, "hooked": 12, "offload_ref": 14}
+RESIDENT = ("llama8b", "cfg0", "small", "mixed", "central", "any")
+HOST = ("streamed", "hooked", "offload_ref", "pageable")
+UPDATE_BYTES = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 20, "central": 14, "any": 34}   # per element, update launch only
+STEP_BYTES = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 24, "central": 16, "any": 34, "streamed": 12, "hooked": 12,
+              "offload_ref": 14, "pageable": 12}
 
 
 # ---- workload shapes -------------------------------------------------------------------------
@@ -163,6 +171,16 @@ def cpu_baseline():
             best = min(best, dt)
     threads = torch.get_num_threads()
     del sets
+    # the same op sequence at config-0 size (one 4096 x 4096 tensor), 1 warm-up pass + best of 5
+    P, G, M, V = (fill_tensor((4096, 4096), kind, 1234 + k, torch.bfloat16, "cpu") for k, kind in enumerate("pgmv"))
+    best0 = float("inf")
+    for it in range(6):
+        t0 = time.perf_counter()
+        torch_ops.reference_step_ops(P, G, M, V, step=10 + it, noise=None, **HP)
+        dt = time.perf_counter() - t0
+        if it:
+            best0 = min(best0, dt)
+    del P, G, M, V
 
     # scalar C restatement, one thread, explicit noise (no RNG cost)
     k = 1 << 22
@@ -177,6 +195,9 @@ def cpu_baseline():
         "sample": f"torch-op restatement of adamw.py:160-222 on CPU tensors, one transformer layer of the set "
                   f"({len(shapes)} tensors, {n} elements), best of 2 passes, {threads} threads, {cpu_model()}",
         "ms_per_sample": best * 1e3,
+        "cfg0_size": {"elements": 4096 * 4096, "ms_per_step": best0 * 1e3, "elements_per_s": 4096 * 4096 / best0,
+                      "algorithmic_GBps": 14 * 4096 * 4096 / best0 / 1e9,
+                      "sample": "the same op sequence on one 4096 x 4096 bf16 tensor, 1 warm-up pass + best of 5"},
         "c_oracle_1thread_elements_per_s": k / c_dt,
     }
 
@@ -235,7 +256,7 @@ def set_states(opt, params, first_step, warmup, dev):
         if pooled and len(params) > 1000:
             continue
         # the states stay the tensors the optimizer allocated (and placed); only their contents are set
-        st["ema"].copy_(fill_tensor(p.shape, "m", 1234 + 4 * i + 2, torch.bfloat16, dev))
+        st["ema"].copy_(fill_tensor(p.shape, "m", 1234 + 4 * i + 2, torch.bfloat16, dev))   # (copy_ widens for wider states)
         st["ema_squared"].copy_(fill_tensor(p.shape, "v", 1234 + 4 * i + 3, st["ema_squared"].dtype, dev))
 
 
@@ -323,6 +344,7 @@ def run_resident(wl, args, steps, warmup, *, full):
     first_step = 100
     opt_kw = dict(storage_device="cuda", seed=1234, state_placement=args.state_placement)
     g_dtype = torch.bfloat16
+    state_dtype = torch.bfloat16
     if wl == "llama8b":
         shapes = llama3_8b_shapes(args.layers)
     elif wl == "central":
@@ -334,13 +356,16 @@ def run_resident(wl, args, steps, warmup, *, full):
     elif wl == "small":
         shapes = small_tensor_shapes()
         opt_kw.update(state_pool_min_bytes=0)   # states as views into two pools, like the large sets
+    elif wl == "any":
+        shapes = llama3_8b_shapes(1)[1:-1]
+        state_dtype = torch.float64
     else:  # mixed
         shapes = llama3_8b_shapes(args.layers)
         g_dtype = torch.float32
         opt_kw.update(loss_scale=1024.0, max_grad_norm=1.0, ema_squared_dtype=torch.float32)
     params, grads, refill_params = build_resident(shapes, g_dtype=g_dtype, device=dev, flat=wl == "small")
     total = sum(numel(s) for s in shapes)
-    opt = ramtorch_amd.AdamW(params, dtype=torch.bfloat16, **HP, **opt_kw)
+    opt = ramtorch_amd.AdamW(params, dtype=state_dtype, **HP, **opt_kw)
     set_states(opt, params, first_step, warmup, dev)
     noise = None
     if wl == "cfg0":
@@ -376,7 +401,8 @@ def run_resident(wl, args, steps, warmup, *, full):
                 "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic[0] if traffic else None,
                 "traffic_source": (f"not measured in this run: rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of an earlier "
                                    f"run, {traffic[1]}") if traffic else None,
-                "kernel": {"mixed": "sr_adamw_fast_wide_kernel", "central": "sr_adamw_fast_kernel (centralizing instance)"}.get(wl, "sr_adamw_fast_kernel"),
+                "kernel": {"mixed": "sr_adamw_fast_wide_kernel", "central": "sr_adamw_fast_kernel (centralizing instance)",
+                           "any": "sr_adamw_any_kernel"}.get(wl, "sr_adamw_fast_kernel"),
                 "kernel_ms": k_ms, "kernel_launches_timed": len(ks), "algorithmic_bytes_per_launch": upd_bytes}
     if settled is not None:
         unsettled = upd_bytes / (settled["kernel_ms_first_batch"] * 1e-3) / 1e9
@@ -395,6 +421,20 @@ def run_resident(wl, args, steps, warmup, *, full):
         out["static_layout"] = {"ms_per_step": ms2, "kernel_ms": sum(ks2) / len(ks2),
                                 "elements_per_s": total / (ms2 * 1e-3), "recorded": opt._frozen is not None}
         opt.unfreeze_layout()
+        # and once with every tensor an allocation of its own (torch's allocator packs them into its
+        # 2 MiB small-tensor blocks at 512-byte steps), as a model's parameters and gradients are
+        sep_p = [torch.nn.Parameter(p.detach().clone(), requires_grad=False) for p in params]
+        for p, g in zip(sep_p, grads):
+            p.grad = g.clone()
+        sep = ramtorch_amd.AdamW(sep_p, dtype=torch.bfloat16, **HP, **dict(opt_kw, state_placement="plain"))
+        for p in sep_p:
+            sep.state[p]["step"] = first_step - 1
+        ms3, ks3 = timed_steps(lambda: sep.step(), max(5, steps // 2), 3, handle, True)
+        k3 = sum(ks3) / len(ks3)
+        out["separate_allocations"] = {"ms_per_step": ms3, "kernel_ms": k3, "achieved": upd_bytes / (k3 * 1e-3) / 1e9,
+                                       "frac": upd_bytes / (k3 * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                                       "note": "one torch allocation per parameter, gradient and state (plain placement)"}
+        del sep, sep_p
     if full:
         # The same state tensors allocated one by one, as the reference allocates them, instead of
         # in two pools placed in different HBM regions: what the placement is worth on this box.
@@ -581,6 +621,66 @@ def run_host(workloads, args, steps, warmup):
     return results
 
 
+def run_pageable(args, steps, warmup):
+    """Parameters and states in ordinary CPU memory (not pinned), gradients on the GPU: a prefix of the
+    Llama-shaped set.  Runs before the large pinned set exists: the bounce buffers are pinned memory, and a
+    process can pin about 64 GiB on the GPU boxes."""
+    import torch
+    import ramtorch_amd
+    from ramtorch_amd.stochastic_optimizers import adamw as adamw_mod
+
+    dev = "cuda:0"
+    shapes, used = [], 0
+    for shp in llama3_8b_shapes(args.layers):
+        if used + 6 * numel(shp) > int(args.pageable_gb * 1e9):
+            break
+        shapes.append(shp)
+        used += 6 * numel(shp)
+    total = sum(numel(s) for s in shapes)
+    params, grads = [], []
+    for i, shp in enumerate(shapes):
+        params.append(torch.nn.Parameter(fill_tensor(shp, "p", 1234 + 4 * i, torch.bfloat16, dev).cpu(), requires_grad=False))
+        grads.append(fill_tensor(shp, "g", 1234 + 4 * i + 1, torch.bfloat16, dev))
+    opt = ramtorch_amd.AdamW(params, dtype=torch.bfloat16, **HP, storage_device="cpu", seed=1234,
+                             stream_chunk_bytes=args.stream_chunk_mb << 20)
+    for i, p in enumerate(params):
+        st = opt.state[p]      # the constructor pins "cpu" states (adamw.py:91-97): these are plain CPU tensors instead
+        st["step"] = 100 - 1 - warmup
+        st["ema"] = fill_tensor(p.shape, "m", 1234 + 4 * i + 2, torch.bfloat16, dev).cpu()
+        st["ema_squared"] = fill_tensor(p.shape, "v", 1234 + 4 * i + 3, torch.bfloat16, dev).cpu()
+        assert not (p.is_pinned() or st["ema"].is_pinned() or st["ema_squared"].is_pinned())
+    gc.collect()
+    _unpin_free_host_blocks()
+    torch.cuda.synchronize()
+    handle = adamw_mod._handle(0)
+    gmap = dict(zip(params, grads))
+    b0 = handle.streamed_bounce_stats()
+    ms_per_step, _ = timed_steps(lambda: opt.step(grads=gmap), steps, warmup, handle, False)
+    b1 = handle.streamed_bounce_stats()
+    link = handle.host_link_probe(args.stream_chunk_mb << 20, reps=8)
+    secs = ms_per_step * 1e-3
+    info = {"h2d_GBps": 6.0 * total / secs / 1e9, "d2h_GBps": 6.0 * total / secs / 1e9,
+            "host_bytes_up": 6.0 * total, "host_bytes_down": 6.0 * total,
+            "bounced_bytes_per_step": (b1["bytes"] - b0["bytes"]) / (steps + warmup),
+            "pinned_h2d_peak_GBps": link["h2d_GBps"], "pinned_d2h_peak_GBps": link["d2h_GBps"],
+            "pinned_duplex_peak_GBps_each_way": link["duplex_GBps_each_way"],
+            "note": "parameters and states in CPU memory that is not pinned: up and down through pinned bounce "
+                    "buffers that host threads fill and empty"}
+    info["h2d_frac_of_peak"] = info["h2d_GBps"] / link["h2d_GBps"]
+    info["frac_of_duplex_peak"] = info["d2h_GBps"] / link["duplex_GBps_each_way"]
+    out = {"ms_per_step": ms_per_step, "elements_per_s": total / secs, "config": config_of("pageable", shapes, total, 100, False),
+           "host_link": info, "roofline": {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                                           "frac": None, "traffic": None, "note": "host-link bound; see host_link"}}
+    del opt, params, grads, gmap
+    gc.collect()
+    torch.cuda.empty_cache()
+    # the handle's bounce buffers (6 GB of pinned memory) go back before the large pinned set is built
+    h = adamw_mod._handles.pop(0, None)
+    if h is not None:
+        h.close()
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -593,6 +693,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=32, help="transformer layers of the Llama-shaped set")
     ap.add_argument("--stream-gb", type=float, default=48.2, help="upper bound on pinned host bytes (host-resident workloads)")
     ap.add_argument("--stream-chunk-mb", type=int, default=256, help="bytes of bf16 per staged chunk and array")
+    ap.add_argument("--pageable-gb", type=float, default=16.0, help="host bytes of the 'pageable' workload (p, ema, ema_squared)")
     ap.add_argument("--state-placement", default="auto", choices=["auto", "plain"],
                     help="AdamW(state_placement=...): 'auto' puts ema and ema_squared into different HBM regions")
     ap.add_argument("--settle-seconds", type=float, default=1.0,
@@ -634,6 +735,8 @@ def main() -> int:
     t_begin = time.perf_counter()
     if wl in RESIDENT:
         main_res = run_resident(wl, args, args.steps, args.warmup, full=True)
+    elif wl == "pageable":
+        main_res = run_pageable(args, args.steps, args.warmup)
     else:
         main_res = run_host([wl], args, args.steps, args.warmup)[wl]
 
@@ -652,7 +755,11 @@ def main() -> int:
         r = run_resident(w, args, k, min(args.warmup, 3), full=False)
         r["steps"] = k
         sec[w] = r
-    host = [w for w in secondary if w in HOST]
+    if "pageable" in secondary:
+        k = max(2, min(args.steps, 3))
+        sec["pageable"] = run_pageable(args, k, 1)
+        sec["pageable"]["steps"] = k
+    host = [w for w in secondary if w in HOST and w != "pageable"]
     if host:
         k = max(2, min(args.steps, 3))
         for w, r in run_host(host, args, k, 1).items():

@@ -1033,6 +1033,9 @@ int rt_row_means_multi(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, fl
         e.row_len = d.row_len;
         e.first_row = (uint32_t)rows;
         e.dtype = (uint32_t)d.g_dtype;
+        if (d.numel / d.row_len > kMaxGrid) return fail(RT_EUNSUPPORTED, "tensor %u: too many rows", i);
+        e.rows = (uint32_t)(d.numel / d.row_len);
+        e.pad[0] = e.pad[1] = e.pad[2] = 0;
         (is_long ? long_tab : tab).push_back(e);
         rows += d.numel / d.row_len;
         if (rows > kMaxGrid) return fail(RT_EUNSUPPORTED, "more than %llu rows in one call", (unsigned long long)kMaxGrid);

@@ -72,20 +72,23 @@ class _HeldBlock:
 
 
 def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: int, *,
-               min_gain: float = 1.05, filler_bytes: int = 2 * GIB, step_bytes: int = 16 * GIB,
-               max_filler_bytes: int = 112 * GIB, max_fraction_of_free: float = 0.5, max_seconds: float = 8.0,
-               log: Optional[Callable[[str], None]] = None):
+               min_gain: float = 1.05, min_gain_anywhere: float = 1.02, filler_bytes: int = 2 * GIB,
+               step_bytes: int = 16 * GIB, max_filler_bytes: int = 112 * GIB, max_fraction_of_free: float = 0.5,
+               max_seconds: float = 1.2, log: Optional[Callable[[str], None]] = None):
     """Two zeroed byte pools on ``device`` such that arrays in the second are, as far as it can be
     arranged, in another HBM region than the corresponding arrays in the first.  Returns
     (pool_a, pool_b, report).
 
-    The place right behind the first pool is tried first.  Unless the probe shows the gain there
-    (at the beginning, in the middle and at the end of the pools alike), memory is occupied with filler blocks
-    (memory the driver hands out in moderate blocks follows in physical address order; one huge
-    block does not) and after every ``step_bytes`` of them the place a block of the pool's size
-    gets is tried, until one shows
-    the gain or the search runs out of ``max_filler_bytes`` (a region is 96 GiB),
-    ``max_fraction_of_free`` of the memory that was free at the start, or ``max_seconds``.
+    The place right behind the first pool is tried first.  A place is taken when the probe shows
+    the gain there: ``min_gain`` on the mean over the beginning, the middle and the end of the pools,
+    and at least ``min_gain_anywhere`` at each of them (in a process that has already allocated and
+    released a lot, a block of many GiB rarely lies in one region from end to end; asking for the full
+    gain everywhere turned such places down and the search ran out of time holding half of the
+    memory).  Otherwise memory is occupied with filler blocks (memory the driver hands out in moderate
+    blocks follows in physical address order; one huge block does not) and after every
+    ``step_bytes`` of them the place a block of the pool's size gets is tried, until one is taken or
+    the search runs out of ``max_filler_bytes`` (a region is 96 GiB), ``max_fraction_of_free`` of the
+    memory that was free at the start, or ``max_seconds`` -- ``report["reason"]`` then says which.
 
     Everything the search occupies on the way -- fillers and the places it tried -- is held through
     the library (``rt_dev_hold``), not through torch, and given back before this returns; the place
@@ -99,20 +102,22 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
         return torch.zeros(nbytes, dtype=torch.uint8, device=device)
 
     t0 = time.monotonic()
-    report = {"placed": False, "filler_GiB": 0.0, "same_GBps": None, "cross_GBps": None, "tries": 0, "seconds": 0.0}
+    report = {"placed": False, "filler_GiB": 0.0, "same_GBps": None, "cross_GBps": None, "tries": 0, "seconds": 0.0,
+              "reason": None}
     free0, _ = torch.cuda.mem_get_info(device)
     a = zeros(bytes_a)
-    budget = min(max_filler_bytes, int(max_fraction_of_free * max(0, free0 - bytes_a - bytes_b)))
+    # (small pools are not worth occupying -- and having the driver clear afterwards -- a hundred GiB for)
+    budget = min(max_filler_bytes, 8 * bytes_b, int(max_fraction_of_free * max(0, free0 - bytes_a - bytes_b)))
     held, held_bytes = [], 0      # addresses of filler blocks held through the library
     best = None                   # (address, same, cross) of the best place seen that fell short of min_gain
     b = None
 
     def summary(r):
-        # mean rates, and whether the gain shows at every probed position (a block that straddles
-        # two regions shows it at some of them only)
+        # mean rates, and whether the place is good enough: the gain on the mean and some gain at every
+        # probed position (a block that straddles two regions shows it at some of them only)
         same = sum(x[0] for x in r) / len(r)
         cross = sum(x[1] for x in r) / len(r)
-        return same, cross, all(x[1] >= min_gain * x[0] for x in r)
+        return same, cross, cross >= min_gain * same and all(x[1] >= min_gain_anywhere * x[0] for x in r)
 
     def adopt(addr, same, cross, placed):
         # this very block becomes the second pool: nothing is released and allocated again
@@ -125,14 +130,17 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
         while b is None:
             free, _ = torch.cuda.mem_get_info(device)
             if bytes_b + 2 * GIB > free:
+                report["reason"] = "not enough free device memory to try another place"
                 break
             try:
                 cand = handle.dev_hold(bytes_b)   # the place the second pool would get right now
             except N.NativeError:
+                report["reason"] = "not enough free device memory to try another place"
                 break
             res = split_probe(handle, a.data_ptr(), bytes_a, cand, bytes_b, device, stream)
             if res is None:                       # pools too small to tell
                 handle.dev_release(cand)
+                report["reason"] = "pools too small for the probe to tell places apart"
                 break
             same, cross, full = summary(res)
             report["tries"] += 1
@@ -155,16 +163,22 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
             else:
                 handle.dev_release(cand)
             free, _ = torch.cuda.mem_get_info(device)
-            if (held_bytes + step_bytes > budget or step_bytes + bytes_b + 4 * GIB > free
-                    or time.monotonic() - t0 > max_seconds):
+            if time.monotonic() - t0 > max_seconds:
+                report["reason"] = f"no place showed the whole gain within {max_seconds:g} s"
+                break
+            if held_bytes + step_bytes > budget or step_bytes + bytes_b + 4 * GIB > free:
+                report["reason"] = (f"no place showed the whole gain with {held_bytes / GIB:.0f} GiB occupied "
+                                    f"(the search may hold {budget / GIB:.0f} GiB)")
                 break
             try:
                 for _ in range(max(1, step_bytes // filler_bytes)):
                     held.append(handle.dev_hold(filler_bytes))
                     held_bytes += filler_bytes
             except N.NativeError:
+                report["reason"] = "not enough free device memory to occupy more"
                 break
         if b is None and best is not None and best[2] >= 1.01 * best[1]:
+            report["reason"] = (report["reason"] or "") + "; the best place seen was taken"
             b = adopt(best[0], best[1], best[2], False)   # part of the gain is better than none
             best = None
     finally:
@@ -174,5 +188,6 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
             handle.dev_release(best[0])
     if b is None:
         b = zeros(bytes_b)
+        report["reason"] = (report["reason"] or "") + "; the second pool is an ordinary allocation"
     report["seconds"] = time.monotonic() - t0
     return a, b, report

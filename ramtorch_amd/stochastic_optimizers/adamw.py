@@ -131,7 +131,9 @@ class AdamW(Optimizer):
             different HBM regions, found by measurement at construction (see
             ``ramtorch_amd/placement.py``; the outcome is in ``state_placement_report``).
             While it searches, the constructor occupies up to half of the free device memory
-            (at most 112 GiB, for at most 8 s) through the library and gives all of it back;
+            (at most 112 GiB and eight times a pool's size, for about a second) through the library and gives all of it back
+            (the driver clears released memory in the background at about 33 GB/s, and until it
+            is done device-wide memory traffic runs about 1 % slower: the first seconds of a run);
             torch's caching allocator only ever sees the first pool (the second is memory held
             through the library, wrapped as a tensor, and released with its last view).
             "plain" allocates every state tensor on its own, as the reference does.

@@ -861,6 +861,35 @@ def test_state_placement_with_most_of_hbm_occupied_falls_back_quietly():
         torch.cuda.empty_cache()
 
 
+def test_state_placement_of_two_large_optimizers_in_a_row():
+    """A process that has allocated and released tens of GiB before (a second model, a second run in one
+    process): the search must still end quickly, and say what it settled for.  Whatever place the states
+    got, the steps are those of an optimizer with plainly allocated states."""
+    n = 1 << 30    # 2 GiB of bf16 per array
+    for round_ in range(2):
+        gen = torch.Generator("cuda").manual_seed(50 + round_)
+        base = (torch.randn(n, device="cuda", generator=gen) * 0.02).bfloat16()
+        grad = (torch.randn(n, device="cuda", generator=gen) * 1e-3).bfloat16()
+        ballast = [torch.empty(8 << 30, dtype=torch.uint8, device="cuda") for _ in range(4 + 2 * round_)]
+        p1 = torch.nn.Parameter(base.clone(), requires_grad=False)
+        p2 = torch.nn.Parameter(base, requires_grad=False)
+        t0 = time.monotonic()
+        opt1 = ramtorch_amd.AdamW([p1], storage_device="cuda", seed=3, state_placement="auto", **HP0)
+        took = time.monotonic() - t0
+        rep = opt1.state_placement_report
+        assert rep is not None and rep["tries"] >= 1, rep
+        assert rep["placed"] or rep["reason"], rep
+        assert rep["seconds"] < 3.0 and took < 4.0, (rep, took)
+        opt2 = ramtorch_amd.AdamW([p2], storage_device="cuda", seed=3, state_placement="plain", **HP0)
+        p1.grad = p2.grad = grad
+        opt1.step(); opt2.step()
+        torch.cuda.synchronize()
+        assert torch.equal(p1.view(torch.int16), p2.view(torch.int16))
+        assert torch.equal(opt1.state[p1]["ema_squared"].view(torch.int16), opt2.state[p2]["ema_squared"].view(torch.int16))
+        del opt1, opt2, p1, p2, base, grad, ballast
+        torch.cuda.empty_cache()       # tens of GiB go back to the driver: the next round starts in a used process
+
+
 def test_frozen_layout_steps_like_the_full_path_and_notices_moved_gradients():
     """assume_static_layout: after the first step the optimizer only checks that parameters and
     gradients are where they were.  Same bits as an optimizer that gathers everything every step,
