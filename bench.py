@@ -11,7 +11,10 @@ workloads, params/states in pinned host memory).  Prints ONE JSON line:
              (wall clock around the steps, device synchronised on both sides)
   roofline   algorithmic HBM bytes per launch / mean kernel time of the update
              kernel, the kernel time taken with HIP events on the launch stream
-             inside the library; peak = 8 TB/s
+             inside the library; peak = 8 TB/s.  ``roofline.settling``: the untimed
+             steps that run before the W warm-up steps until the driver has finished
+             clearing the device memory that set-up released (see ``settle``), with
+             the kernel time of every batch of them
   secondary  the other configurations, each measured the same way in the same
              process with fewer steps (only when the main workload is the
              default one; ``--secondary none`` leaves them out)
@@ -29,7 +32,7 @@ ema~N(0,1e-4), ema_squared=N(0,1e-3)^2, stored bf16):
   mixed     Llama-3-8B shapes; bf16 p and ema, fp32 ema_squared, fp32 grads scaled
             by 1024 and unscaled in-kernel, global-norm clip to 1.0
   central   the default set with centralization=1.0 (adamw.py:179-184): one row-mean
-            pass per tensor (2 B per element read) and the update through the fast
+            pass over all gradients (2 B per element read) and the update through the fast
             kernel's instance that subtracts the means (14 B per element + 4 B per row)
   streamed  Llama-3-8B shapes with p/ema/ema_squared in pinned host memory,
             bf16 grads on the GPU, 256 MB chunks (--stream-gb bounds the host set)
@@ -334,6 +337,47 @@ def config_of(wl, shapes, total, first_step, explicit):
                         "weight_decay": HP["weight_decay"]}}
 
 
+def class_table(opt, params, grads, handle):
+    """The update kernel's rate per shape class of the Llama-shaped set, on the tensors where the bench and
+    the optimizer put them: five steps over the tensors of each class alone (kernel time from the
+    library's events), and afterwards the math-free probe of the same traffic on one tensor of the class
+    with its gradient and its two states (the probe overwrites what it runs on)."""
+    import torch
+    layer = lambda l, k: 1 + 9 * l + k
+    classes = {"embed, lm_head (128256x4096)": [0, 289],
+               "q, o (4096x4096)": [layer(l, k) for l in range(32) for k in (0, 3)],
+               "k, v (1024x4096)": [layer(l, k) for l in range(32) for k in (1, 2)],
+               "gate, up (14336x4096)": [layer(l, k) for l in range(32) for k in (4, 5)],
+               "down (4096x14336)": [layer(l, 6) for l in range(32)]}
+    out = {}
+    for name, idx in classes.items():
+        gm = {params[i]: grads[i] for i in idx}
+        for p in params:
+            p.grad = None
+        opt.step(grads=gm)
+        torch.cuda.synchronize()
+        handle.set_timing(True)
+        for _ in range(5):
+            opt.step(grads=gm)
+        torch.cuda.synchronize()
+        ks = handle.kernel_ms_history(5)
+        handle.set_timing(False)
+        n = sum(params[i].numel() for i in idx)
+        ms = sum(ks) / len(ks)
+        out[name] = {"tensors": len(idx), "elements": n, "kernel_ms": ms, "achieved": 14 * n / (ms * 1e-3) / 1e9,
+                     "frac": 14 * n / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+    for name, idx in classes.items():
+        rates = []
+        for i in (idx[0], idx[len(idx) // 2], idx[-1]):
+            st = opt.state[params[i]]
+            n = params[i].numel() // 8192 * 8192
+            ms = handle.stream_probe(params[i].data_ptr(), grads[i].data_ptr(), st["ema"].data_ptr(),
+                                     st["ema_squared"].data_ptr(), n, reps=max(5, int(3e8 // n)))
+            rates.append(14 * n / (ms * 1e-3) / 1e9)
+        out[name]["probe_GBps_first_middle_last_tensor"] = rates
+    return out
+
+
 def run_resident(wl, args, steps, warmup, *, full):
     """One resident workload.  ``full``: also the math-free ceilings and the plain-placement comparison."""
     import torch
@@ -388,7 +432,7 @@ def run_resident(wl, args, steps, warmup, *, full):
         # the device runs under the workload's own load until its clocks have settled; then parameters
         # and states are drawn again (same seeds, same distributions) and the step counts put back,
         # so that the timed steps start from the configuration's inputs at the configuration's step
-        settled = settle(one_step, handle, args.settle_seconds, args.settle_max_seconds)
+        settled = settle(one_step, handle, args.settle_seconds, args.settle_max_seconds if full else min(args.settle_max_seconds, 4.0))
         refill_params()
         set_states(opt, params, first_step, warmup, dev)
         torch.cuda.synchronize()
@@ -447,6 +491,8 @@ def run_resident(wl, args, steps, warmup, *, full):
             roofline["plain_placement"] = {"kernel_ms": k2, "achieved": upd_bytes / (k2 * 1e-3) / 1e9,
                                            "frac": upd_bytes / (k2 * 1e-3) / 1e9 / HBM_PEAK_GBPS}
             del plain
+        if args.class_table and wl == "llama8b" and args.layers == 32:
+            roofline["classes"] = class_table(opt, params, grads, handle)
         # What the same traffic pattern reaches with the arithmetic removed (the all-bf16 pattern:
         # 8 B read + 6 B written per element).  Where the arrays lie in HBM matters, so it is measured
         # twice: on four fresh buffers allocated side by side, and on the workload's own largest
@@ -700,7 +746,10 @@ def main() -> int:
                     help="resident workloads: untimed steps for at least this long before the warm-up steps, and on "
                          "until the driver has finished clearing released device memory in the background (a step "
                          "gets 0.6 %% faster) or --settle-max-seconds have passed (0 = no such steps)")
-    ap.add_argument("--settle-max-seconds", type=float, default=6.0)
+    ap.add_argument("--settle-max-seconds", type=float, default=8.0,
+                    help="upper bound of that phase for the main workload (the secondary ones: at most 4 s)")
+    ap.add_argument("--class-table", action="store_true",
+                    help="llama8b: also the kernel's rate and the math-free probe's per shape class of the set")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pmc-calibrate", action="store_true",
                     help="also launch one plain elementwise kernel that reads 1 GiB and writes 1 GiB, so that "
