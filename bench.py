@@ -428,6 +428,13 @@ def run_resident(wl, args, steps, warmup, *, full):
 
     one_step = lambda: opt.step(noise=noise, grads=gmap)
     settled = None
+    if args.release_gib > 0 and full:
+        # diagnostic: take this much device memory from the driver and give it straight back, so that the
+        # settling steps below run while the driver clears it (their kernel times show for how long)
+        time.sleep(max(0.0, args.idle_before_release))
+        held = [handle.dev_hold(2 << 30) for _ in range(int(args.release_gib // 2))]
+        for addr in held:
+            handle.dev_release(addr)
     if args.settle_seconds > 0:
         # the device runs under the workload's own load until its clocks have settled; then parameters
         # and states are drawn again (same seeds, same distributions) and the step counts put back,
@@ -748,6 +755,11 @@ def main() -> int:
                          "gets 0.6 %% faster) or --settle-max-seconds have passed (0 = no such steps)")
     ap.add_argument("--settle-max-seconds", type=float, default=8.0,
                     help="upper bound of that phase for the main workload (the secondary ones: at most 4 s)")
+    ap.add_argument("--release-gib", type=float, default=0.0,
+                    help="diagnostic (main workload): hold and release this much device memory right before the "
+                         "settling steps, to see what the driver's background clearing of it costs and for how long")
+    ap.add_argument("--idle-before-release", type=float, default=6.0,
+                    help="with --release-gib: idle this long first, so that what set-up released has been cleared")
     ap.add_argument("--class-table", action="store_true",
                     help="llama8b: also the kernel's rate and the math-free probe's per shape class of the set")
     ap.add_argument("--no-cpu-baseline", action="store_true")
