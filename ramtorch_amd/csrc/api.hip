@@ -492,9 +492,8 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
             const DevTensor& t = tens[k];
             const uint32_t nc = (uint32_t)((t.numel + kChunkElems - 1) / kChunkElems);
             uint32_t j0 = 0;
-            constexpr uint32_t chunks_per_unit = kFastUnitElems / kChunkElems;
-            if (plain(t)) j0 = has_pieces ? nc : (uint32_t)(t.numel / unit) * chunks_per_unit;
-            if (cen_plain(t)) j0 = (uint32_t)(t.numel / unit) * chunks_per_unit;
+            if (plain(t)) j0 = has_pieces ? nc : (uint32_t)((t.numel / unit) * unit / kChunkElems);
+            if (cen_plain(t)) j0 = (uint32_t)((t.numel / unit) * unit / kChunkElems);
             for (uint32_t j = j0; j < nc; ++j) chunks.push_back(ChunkRef{(uint32_t)k, j});
         }
         b.n_generic = (uint32_t)chunks.size() - b.first_generic;
