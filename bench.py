@@ -116,16 +116,25 @@ def numel(shape):
     return n
 
 
+_FILL_SCRATCH = {}
+
+
 def fill_tensor(shape, kind: str, seed: int, dtype, device):
-    """Synthetic values of one array, drawn in fp32 on `device` and stored as `dtype`."""
+    """Synthetic values of one array, drawn in fp32 on `device` and stored as `dtype`.  The fp32 values
+    are drawn into one scratch buffer per device that is allocated once, before anything else: the
+    tensors of a set then follow each other in device memory as a model's do, instead of landing in
+    whatever blocks earlier temporaries left behind in torch's allocator."""
     import torch
     gen = torch.Generator(device=device).manual_seed(seed)
     n = numel(shape)
+    step = 1 << 28  # bound the fp32 scratch
+    scratch = _FILL_SCRATCH.get(str(device))
+    if scratch is None:
+        scratch = _FILL_SCRATCH[str(device)] = torch.empty(step, dtype=torch.float32, device=device)
     out = torch.empty(n, dtype=dtype, device=device)
-    step = 1 << 28  # bound the fp32 temporary
     for lo in range(0, n, step):
         k = min(step, n - lo)
-        x = torch.randn(k, device=device, generator=gen)
+        x = scratch[:k].normal_(generator=gen)
         if kind == "p":
             x.mul_(0.02)
         elif kind == "g":
