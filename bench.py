@@ -85,8 +85,8 @@ HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
 METRIC = "SR-AdamW step: params/sec + achieved HBM GB/s (% of peak), 8B bf16 set, 1 GPU"
 RESIDENT = ("llama8b", "cfg0", "small", "mixed", "central", "any")
 HOST = ("streamed", "hooked", "offload_ref", "pageable")
-UPDATE_BYTES = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 20, "central": 14, "any": 34}   # per element, update launch only
-STEP_BYTES = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 24, "central": 16, "any": 34, "streamed": 12, "hooked": 12,
+UPDATE_BYTES = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 20, "central": 14, "any": 38}   # per element, update launch only
+STEP_BYTES = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 24, "central": 16, "any": 38, "streamed": 12, "hooked": 12,
               "offload_ref": 14, "pageable": 12}
 
 
