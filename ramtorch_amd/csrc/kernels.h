@@ -902,7 +902,10 @@ __device__ __forceinline__ void store8_any(uint64_t base, uint32_t dt, uint64_t 
 // shared memory that belong to this wave alone: written in array order, read back as each lane's own
 // eight consecutive elements.  A wave's shared-memory instructions execute in the order issued, so
 // no barrier is needed; the fences only keep the compiler from moving them across each other.
-// fp64 state layouts ran at 4.4 TB/s with per-lane accesses.
+// fp64 state layouts ran at 4.4 TB/s with per-lane accesses.  (Issuing the loads of all four arrays
+// before the first of them is unpacked, each array with a stage of its own, needs 153 registers --
+// three waves per SIMD instead of four -- and ran 1 - 10 % slower on every layout; fetching the next
+// 512 elements ahead of the arithmetic as well needs 255.)
 __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
