@@ -50,12 +50,22 @@ def bits32(t):
 
 def run_both(handle, p, g, m, v, *, hp=HP0, step=10, noise=None, seed=1234, tensor_id=0, debug=True,
              g_dtype=oracle.DT_BF16, p_dtype=oracle.DT_BF16, m_dtype=oracle.DT_BF16, v_dtype=oracle.DT_BF16,
-             inv_loss_scale=1.0, clip_coef=None):
-    """One tensor through the HIP library and through the oracle; returns both result sets."""
+             inv_loss_scale=1.0, clip_coef=None, pad=0):
+    """One tensor through the HIP library and through the oracle; returns both result sets.
+    pad: the arrays are the first elements of allocations that many elements longer, and what lies
+    behind them has to be the same afterwards."""
     tdt = {oracle.DT_BF16: torch.bfloat16, oracle.DT_F16: torch.float16}
+    padded = []
 
     def up(a, code):
-        return torch.from_numpy(a.copy()).cuda() if code in (oracle.DT_F32, oracle.DT_F64) else dev16(a, tdt[code])
+        t = torch.from_numpy(a.copy()).cuda() if code in (oracle.DT_F32, oracle.DT_F64) else dev16(a, tdt[code])
+        if pad:
+            whole = torch.empty(a.size + pad, dtype=t.dtype, device="cuda")
+            whole.view(torch.uint8).fill_(0xA5)
+            whole[:a.size] = t
+            padded.append(whole)
+            t = whole[:a.size]
+        return t
 
     P, G, M, V = up(p, p_dtype), up(g, g_dtype), up(m, m_dtype), up(v, v_dtype)
     n = p.size
@@ -66,6 +76,8 @@ def run_both(handle, p, g, m, v, *, hp=HP0, step=10, noise=None, seed=1234, tens
     coef_t = None if clip_coef is None else torch.tensor([clip_coef], dtype=torch.float32, device="cuda")
     F.step_resident(handle, [e], [sc], seed=seed, explicit_noise=noise is not None, clip_coef=coef_t)
     torch.cuda.synchronize()
+    for whole in padded:
+        assert bool((whole[n:].view(torch.uint8) == 0xA5).all()), "bytes behind the tensor were written"
 
     po, mo, vo = p.copy(), m.copy(), v.copy()
     sco = oracle.scalars_from_hparams(step=step, inv_loss_scale=inv_loss_scale, apply_clip=clip_coef is not None, **hp)
@@ -243,6 +255,33 @@ def test_dtype_combinations(handle, p_dt, g_dt, m_dt, v_dt, mode):
         got, want, dbg, pre = run_both(handle, p, g, m, v, noise=noise, p_dtype=p_dt, g_dtype=g_dt, m_dtype=m_dt,
                                        v_dtype=v_dt, debug=debug)
         assert_same(got, want, dbg, pre, f"dtypes {p_dt}{g_dt}{m_dt}{v_dt} {mode}")
+
+
+@pytest.mark.parametrize("n", [8, 504, 511, 512, 513, 520, 1024, 2047, 2048, 2056, 8192, 8192 + 512, 8192 + 519, 3 * 8192 - 1])
+def test_runtime_typed_kernel_around_a_wavefronts_run(handle, n):
+    """The runtime-typed kernel moves fp32 and fp64 arrays a whole wavefront (512 elements) at a time where
+    all 512 exist and lane by lane behind that: sizes on both sides of those edges, the three wide
+    layouts, both noise modes, and the memory behind the arrays has to stay as it was."""
+    for p_dt, g_dt, m_dt, v_dt in [(oracle.DT_BF16, oracle.DT_BF16, oracle.DT_F64, oracle.DT_F64),
+                                   (oracle.DT_F64, oracle.DT_F32, oracle.DT_F32, oracle.DT_F64),
+                                   (oracle.DT_F16, oracle.DT_BF16, oracle.DT_F64, oracle.DT_F32)]:
+        p, g, m, v = oracle.synth_inputs(n, 100 + n)
+
+        def conv(a, dt):
+            f = oracle.bf16_to_f32(a)
+            if dt == oracle.DT_F32:
+                return (f * np.float32(1.0009765625)).astype(np.float32)
+            if dt == oracle.DT_F16:
+                return f.astype(np.float16).view(np.uint16)
+            if dt == oracle.DT_F64:
+                return f.astype(np.float64) * (1.0 + 2.0 ** -30)
+            return a
+        for mode in ("philox", "explicit"):
+            noise = oracle.synth_noise(n, 7) if mode == "explicit" else None
+            got, want, dbg, pre = run_both(handle, conv(p, p_dt), conv(g, g_dt), conv(m, m_dt), conv(v, v_dt), noise=noise,
+                                           p_dtype=p_dt, g_dtype=g_dt, m_dtype=m_dt, v_dtype=v_dt, debug=False, step=3,
+                                           pad=1024)
+            assert_same(got, want, dbg, pre, f"n={n} dtypes {p_dt}{g_dt}{m_dt}{v_dt} {mode}")
 
 
 def test_fp16_param_overflow_and_gradual_underflow(handle):
