@@ -80,6 +80,7 @@ OFFLINE_TRAFFIC = {
     "small": (1_090_935_301, _TRAFFIC_FILE),
     "cfg0": (335_774_529, _TRAFFIC_FILE),
     "central": (112_473_148_416 + 3_860_685, _TRAFFIC_FILE),   # centralizing fast instance + generic kernel for the norm vectors
+    "any": (8_292_259_533, _TRAFFIC_FILE),
 }
 HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
 METRIC = "SR-AdamW step: params/sec + achieved HBM GB/s (% of peak), 8B bf16 set, 1 GPU"
@@ -448,7 +449,7 @@ def run_resident(wl, args, steps, warmup, *, full):
         # the device runs under the workload's own load until its clocks have settled; then parameters
         # and states are drawn again (same seeds, same distributions) and the step counts put back,
         # so that the timed steps start from the configuration's inputs at the configuration's step
-        settled = settle(one_step, handle, args.settle_seconds, args.settle_max_seconds if full else min(args.settle_max_seconds, 4.0))
+        settled = settle(one_step, handle, args.settle_seconds, args.settle_max_seconds if full else min(args.settle_max_seconds, 6.0))
         refill_params()
         set_states(opt, params, first_step, warmup, dev)
         torch.cuda.synchronize()
@@ -763,7 +764,7 @@ def main() -> int:
                          "until the driver has finished clearing released device memory in the background (a step "
                          "gets 0.6 %% faster) or --settle-max-seconds have passed (0 = no such steps)")
     ap.add_argument("--settle-max-seconds", type=float, default=8.0,
-                    help="upper bound of that phase for the main workload (the secondary ones: at most 4 s)")
+                    help="upper bound of that phase for the main workload (the secondary ones: at most 6 s)")
     ap.add_argument("--release-gib", type=float, default=0.0,
                     help="diagnostic (main workload): hold and release this much device memory right before the "
                          "settling steps, to see what the driver's background clearing of it costs and for how long")
