@@ -131,7 +131,7 @@ class AdamW(Optimizer):
             different HBM regions, found by measurement at construction (see
             ``ramtorch_amd/placement.py``; the outcome is in ``state_placement_report``).
             While it searches, the constructor occupies up to half of the free device memory
-            (at most 112 GiB and eight times a pool's size, for about a second) through the library and gives all of it back
+            (at most 112 GiB, for pools under 1 GiB eight times their size; for about a second) through the library and gives all of it back
             (the driver clears released memory in the background at about 33 GB/s, and until it
             is done device-wide memory traffic runs about 1 % slower: the first seconds of a run);
             torch's caching allocator only ever sees the first pool (the second is memory held
@@ -891,6 +891,10 @@ class AdamW(Optimizer):
             raise NotImplementedError("step_param with max_grad_norm (the global norm needs every gradient)")
         if id(p) in self._stepped_early:
             raise RuntimeError("step_param called twice for one parameter without a step() in between")
+        if self.__dict__.get("_frozen") is not None:
+            # a recorded layout does not cover steps of single parameters, and while it is in use the
+            # step counts in the states lag: bring them up to date before one of them is read
+            self.unfreeze_layout()
         recs = self._records()
         pos = self._positions.get(id(p))
         if pos is None:

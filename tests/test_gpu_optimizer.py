@@ -959,6 +959,16 @@ def test_frozen_layout_steps_like_the_full_path_and_notices_moved_gradients():
     a.unfreeze_layout()
     assert [a.state[p]["step"] for p in ps_a] == [b.state[p]["step"] for p in ps_b]
     a.step(); b.step(); same()
+    # one parameter stepped on its own while a layout is recorded and its step counts lag
+    a.step(); b.step(); same()
+    assert a._frozen is not None
+    a.step(); b.step(); same()
+    assert a._frozen["pending"] >= 1
+    for opt, ps in ((a, ps_a), (b, ps_b)):
+        opt.step_param(ps[2])
+        opt.step()
+    same()
+    assert [a.state[p]["step"] for p in ps_a] == [b.state[p]["step"] for p in ps_b]
 
 
 @pytest.mark.parametrize("shape", [(37, 24), (4, 3, 10), (129,)])
