@@ -31,9 +31,10 @@ ema~N(0,1e-4), ema_squared=N(0,1e-3)^2, stored bf16):
   small     20 000 small tensors (length log-uniform in [1,4096]) + 64 x 1024x1024
   mixed     Llama-3-8B shapes; bf16 p and ema, fp32 ema_squared, fp32 grads scaled
             by 1024 and unscaled in-kernel, global-norm clip to 1.0
-  central   the default set with centralization=1.0 (adamw.py:179-184): one row-mean
-            pass over all gradients (2 B per element read) and the update through the fast
-            kernel's instance that subtracts the means (14 B per element + 4 B per row)
+  central   the default set with centralization=1.0 (adamw.py:179-184): one launch in which a
+            wavefront sums a gradient row and then updates it (14 B per element from HBM; the
+            row is read a second time out of the L2); next to it the same steps with a row-mean
+            pass of their own first (16 B per element)
   streamed  Llama-3-8B shapes with p/ema/ema_squared in pinned host memory,
             bf16 grads on the GPU, 256 MB chunks (--stream-gb bounds the host set)
   hooked    the same set, but each tensor is updated by AdamW.step_param() as a
@@ -79,7 +80,7 @@ OFFLINE_TRAFFIC = {
     "mixed": (160_597_606_615, _TRAFFIC_FILE),      # the update launch; its norm pass fetches 32 120 545 889 B more
     "small": (1_090_935_301, _TRAFFIC_FILE),
     "cfg0": (335_774_529, _TRAFFIC_FILE),
-    "central": (112_473_148_416 + 3_860_685, _TRAFFIC_FILE),   # centralizing fast instance + generic kernel for the norm vectors
+    "central": (116_177_807_872, _TRAFFIC_FILE),   # row-wise kernel: every gradient row read twice, 77 % of the second reads out of the L2
     "any": (8_292_259_533, _TRAFFIC_FILE),
 }
 HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
@@ -87,7 +88,7 @@ METRIC = "SR-AdamW step: params/sec + achieved HBM GB/s (% of peak), 8B bf16 set
 RESIDENT = ("llama8b", "cfg0", "small", "mixed", "central", "any")
 HOST = ("streamed", "hooked", "offload_ref", "pageable")
 UPDATE_BYTES = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 20, "central": 14, "any": 38}   # per element, update launch only
-STEP_BYTES = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 24, "central": 16, "any": 38, "streamed": 12, "hooked": 12,
+STEP_BYTES = {"llama8b": 14, "small": 14, "cfg0": 20, "mixed": 24, "central": 14, "any": 38, "streamed": 12, "hooked": 12,
               "offload_ref": 14, "pageable": 12}
 
 
@@ -462,7 +463,7 @@ def run_resident(wl, args, steps, warmup, *, full):
                 "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic[0] if traffic else None,
                 "traffic_source": (f"not measured in this run: rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of an earlier "
                                    f"run, {traffic[1]}") if traffic else None,
-                "kernel": {"mixed": "sr_adamw_fast_wide_kernel", "central": "sr_adamw_fast_kernel (centralizing instance)",
+                "kernel": {"mixed": "sr_adamw_fast_wide_kernel", "central": "sr_adamw_rowwise_kernel",
                            "any": "sr_adamw_any_kernel"}.get(wl, "sr_adamw_fast_kernel"),
                 "kernel_ms": k_ms, "kernel_launches_timed": len(ks), "algorithmic_bytes_per_launch": upd_bytes}
     if settled is not None:
@@ -531,6 +532,16 @@ def run_resident(wl, args, steps, warmup, *, full):
         roofline["frac_of_pattern_ceiling"] = (achieved / roofline["pattern_ceiling_GBps"]
                                                if wl in ("llama8b", "small") else None)
     roofline["state_placement"] = {"mode": args.state_placement, **(opt.state_placement_report or {})}
+    if wl == "central":
+        # the same steps with the row means taken by a pass of their own first (what tensors whose rows do
+        # not fit a wavefront get): 2 B per element more from HBM and one launch more
+        opt.fuse_row_means = False
+        ms2, ks2 = timed_steps(one_step, max(3, steps // 4), 2, handle, True)
+        k2 = sum(ks2) / len(ks2)
+        opt.fuse_row_means = True
+        roofline["separate_row_mean_pass"] = {
+            "ms_per_step": ms2, "update_kernel_ms": k2, "row_mean_pass_ms": ms2 - k2,
+            "note": "row_mean_table_kernel (16.06 GB read) + the fast kernel's centralizing instance, 16 B per element"}
     if wl == "mixed":
         # the norm pass is a launch of its own (4 B per element read); time it apart
         from ramtorch_amd import functional as F

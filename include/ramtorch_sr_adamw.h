@@ -84,10 +84,15 @@ typedef struct rt_tensor_desc {
     float* dbg_m;
     float* dbg_v;
     const float* row_mean; /* centralization != 0: device fp32[numel/row_len] row means of g (of the unscaled,
-                              unclipped gradient: a clip coefficient is applied to the mean as to the gradient) */
+                              unclipped gradient: a clip coefficient is applied to the mean as to the gradient).
+                              NULL with row_len set (rt_step_multi only): the update kernel takes the row means
+                              itself -- same summation, same bits as rt_row_means -- which saves the separate pass
+                              over g; for whole tensors (elem_offset 0, numel a multiple of row_len) of 16-bit
+                              arrays, 16-byte aligned, Philox noise, no debug outputs, row_len a multiple of 8
+                              in [512, 32768]; RT_EINVAL otherwise */
     uint64_t numel;
     uint64_t elem_offset;  /* index of element 0 inside the logical tensor; multiple of 8 */
-    uint64_t row_len;      /* elements per row (dim 0 slice) when row_mean != NULL */
+    uint64_t row_len;      /* elements per row (dim 0 slice) when centralization != 0 */
     uint32_t tensor_id;    /* < 2^30; part of the Philox counter */
     uint32_t step;         /* state["step"] after the increment (adamw.py:177), mod 2^32 */
     uint32_t scalars_idx;  /* index into the rt_scalars array */

@@ -140,6 +140,7 @@ struct Batch {            // tensors of one dtype combination inside a table ima
     uint32_t first_piece, n_pieces;            // pieces served by the fast kernel's first workgroups
     uint32_t first_generic, n_generic;         // chunk range of the generic kernel
     uint32_t first_cen_range, n_cen_ranges, n_cen_units;  // the same lists for tensors with centralization
+    uint32_t first_rw_range, n_rw_ranges, n_rw_rows;      // tensors whose row means the kernel takes itself: first rows
 };
 
 struct Plan {
@@ -250,6 +251,7 @@ struct KernelPair {
     MultiKernel fast;     // whole fast units of aligned tensors, plus (16-bit layouts, Philox) their pieces
     MultiKernel generic;  // unaligned tensors, debug outputs, leftovers without a piece path, rows shorter than 8
     MultiKernel fast_cen; // whole fast units of aligned tensors with centralization (16-bit layouts, Philox), or NULL
+    MultiKernel rowwise;  // whole tensors with centralization whose row means the kernel takes itself (same layouts), or NULL
 };
 
 template <int P, int G, int M, int V>
@@ -259,15 +261,15 @@ static KernelPair pick_noise(int noise) {
     if constexpr (wide) {
         if (noise == RT_NOISE_EXPLICIT)
             return {sr_adamw_fast_wide_kernel<P, G, M, V, RT_NOISE_EXPLICIT>,
-                    sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_EXPLICIT>, nullptr};
+                    sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_EXPLICIT>, nullptr, nullptr};
         return {sr_adamw_fast_wide_kernel<P, G, M, V, RT_NOISE_PHILOX>,
-                sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_PHILOX>, nullptr};
+                sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_PHILOX>, nullptr, nullptr};
     } else {
         if (noise == RT_NOISE_EXPLICIT)
             return {sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_EXPLICIT>,
-                    sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_EXPLICIT>, nullptr};
+                    sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_EXPLICIT>, nullptr, nullptr};
         return {sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_PHILOX>, sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_PHILOX>,
-                sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_PHILOX, true>};
+                sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_PHILOX, true>, sr_adamw_rowwise_kernel<P, G, M, V>};
     }
 }
 // State dtype pairs the templated kernels are instantiated for: every bf16 / fp32 mix, and both fp16.
@@ -312,6 +314,17 @@ static inline bool compiled_combo(const rt_tensor_desc& d) {
 // Launch group of a tensor: its dtype combination when the templated kernels cover it.
 static inline uint32_t combo_of(const rt_tensor_desc& d) { return compiled_combo(d) ? dtypes_of(d) : kComboAny; }
 
+// Centralization with row_mean == NULL: whether the row-wise kernel can take this tensor
+// (see sr_adamw_rowwise_kernel).
+static inline bool rowwise_ok(const rt_tensor_desc& d, int noise_mode, bool allow_host) {
+    const uintptr_t all = (uintptr_t)d.p | (uintptr_t)d.g | (uintptr_t)d.m | (uintptr_t)d.v;
+    return !allow_host && noise_mode == RT_NOISE_PHILOX && compiled_combo(d) && d.p_dtype != RT_DT_F32 &&
+           d.g_dtype != RT_DT_F32 && d.m_dtype != RT_DT_F32 && d.v_dtype != RT_DT_F32 && (all & 15u) == 0 &&
+           !d.dbg_p && !d.dbg_m && !d.dbg_v && d.elem_offset == 0 && d.row_len % kVec == 0 &&
+           d.row_len >= kRowwiseMinLen && d.row_len <= kWaveRowMax && d.numel % d.row_len == 0 &&
+           d.numel / d.row_len <= kMaxGrid;
+}
+
 // ---------------------------------------------------------------------------
 // argument validation shared by the resident and streamed entry points
 // ---------------------------------------------------------------------------
@@ -353,8 +366,13 @@ static int validate(const rt_tensor_desc* descs, uint32_t n, const rt_scalars* s
                 return fail(RT_EINVAL, "tensor %u: explicit noise missing for a bf16 array", i);
         }
         if (scalars[d.scalars_idx].centralization != 0.0f) {
-            if (!d.row_mean || d.row_len == 0)
-                return fail(RT_EINVAL, "tensor %u: centralization without row_mean/row_len", i);
+            if (d.row_len == 0) return fail(RT_EINVAL, "tensor %u: centralization without row_len", i);
+            if (!d.row_mean && !rowwise_ok(d, noise_mode, allow_host))
+                return fail(RT_EINVAL,
+                            "tensor %u: centralization without row_mean (the update takes the row means itself only "
+                            "for whole 16-byte-aligned device tensors of 16-bit arrays with Philox noise, rows a "
+                            "multiple of 8 and %u .. %u elements long, no debug outputs)",
+                            i, kRowwiseMinLen, kWaveRowMax);
         }
     }
     return RT_OK;
@@ -415,6 +433,7 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
         t.dtypes = dtypes_of(d);
         const uint64_t all = t.p | t.g | t.m | t.v | t.np | t.nm | t.nv;
         t.flags = (all & 15u) == 0 ? kFlagAligned : 0u;
+        if (sets[it->second].s.centralization != 0.0f && !d.row_mean) t.flags |= kFlagRowwise;   // validated: rowwise_ok
     }
 
     // ---- work lists, combination by combination
@@ -439,7 +458,8 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
         b.first_piece = (uint32_t)pieces.size();
         const bool has_pieces = !want_explicit && narrow_combo(combo);
         auto plain = [&](const DevTensor& t) {
-            return combo != kComboAny && (t.flags & kFlagAligned) && (t.dp | t.dm | t.dv | t.row_mean) == 0;
+            return combo != kComboAny && (t.flags & kFlagAligned) && !(t.flags & kFlagRowwise) &&
+                   (t.dp | t.dm | t.dv | t.row_mean) == 0;
         };
         uint32_t units = 0;
         for (size_t k = k0; k < k1; ++k) {
@@ -487,6 +507,18 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
         }
         b.n_cen_ranges = (uint32_t)ranges.size() - b.first_cen_range;
         b.n_cen_units = cen_units;
+        // Tensors whose row means the update takes itself: whole tensors, a wavefront per row.
+        b.first_rw_range = (uint32_t)ranges.size();
+        uint64_t rw_rows = 0;
+        for (size_t k = k0; k < k1; ++k) {
+            const DevTensor& t = tens[k];
+            if (!(t.flags & kFlagRowwise)) continue;
+            ranges.push_back((uint32_t)rw_rows);
+            fast_tens.push_back(t);
+            rw_rows += t.numel / t.row_len;
+        }
+        b.n_rw_ranges = (uint32_t)ranges.size() - b.first_rw_range;
+        b.n_rw_rows = (uint32_t)std::min<uint64_t>(rw_rows, 0xFFFFFFFFull);   // checked against the grid limit at launch
         b.first_generic = (uint32_t)chunks.size();
         for (size_t k = k0; k < k1; ++k) {
             const DevTensor& t = tens[k];
@@ -494,6 +526,7 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
             uint32_t j0 = 0;
             if (plain(t)) j0 = has_pieces ? nc : (uint32_t)((t.numel / unit) * unit / kChunkElems);
             if (cen_plain(t)) j0 = (uint32_t)((t.numel / unit) * unit / kChunkElems);
+            if (t.flags & kFlagRowwise) j0 = nc;
             for (uint32_t j = j0; j < nc; ++j) chunks.push_back(ChunkRef{(uint32_t)k, j});
         }
         b.n_generic = (uint32_t)chunks.size() - b.first_generic;
@@ -595,7 +628,7 @@ static int enqueue_kernels(const Plan& plan, const uint8_t* base, uint64_t seed,
     };
     std::vector<Launch> launches;
     for (const Batch& b : plan.batches) {
-        KernelPair k;
+        KernelPair k{};
         if (b.combo == kComboAny) {
             k.fast = nullptr;  // no ranges and no pieces for this group
             k.generic = noise_mode == RT_NOISE_EXPLICIT ? sr_adamw_any_kernel<RT_NOISE_EXPLICIT>
@@ -625,6 +658,19 @@ static int enqueue_kernels(const Plan& plan, const uint8_t* base, uint64_t seed,
             c.n_ranges = b.n_cen_ranges;
             c.n_pieces = c.n_piece_wgs = c.piece_rate = 0;
             launches.push_back(Launch{k.fast_cen, b.n_cen_units, c});
+        }
+        if (b.n_rw_rows) {
+            if (!k.rowwise) return fail(RT_EHIP, "internal: row-wise tensors without a kernel for them");
+            const uint64_t rw_grid = ((uint64_t)b.n_rw_rows + kThreads / 64 - 1) / (kThreads / 64);
+            if (b.n_rw_rows == 0xFFFFFFFFu || rw_grid > kMaxGrid)
+                return fail(RT_EUNSUPPORTED, "too many rows in one launch");
+            LaunchArgs c = a;
+            c.first = (const uint32_t*)(base + plan.off_ranges) + b.first_rw_range;
+            c.fast_tensors = (const DevTensor*)(base + plan.off_fast_tensors) + b.first_rw_range;
+            c.n_ranges = b.n_rw_ranges;
+            c.n_rows = b.n_rw_rows;
+            c.n_pieces = c.n_piece_wgs = c.piece_rate = 0;
+            launches.push_back(Launch{k.rowwise, (uint32_t)rw_grid, c});
         }
     }
     for (size_t i = 0; i < launches.size(); ++i) {

@@ -14,6 +14,7 @@ constexpr uint32_t kChunkElems = kThreads * kVec * kItersPerChunk;  // 8192
 
 // DevTensor.flags
 constexpr uint32_t kFlagAligned = 1u;  // every array pointer of the tensor is 16-byte aligned
+constexpr uint32_t kFlagRowwise = 2u;  // centralization with the row means taken inside the update kernel (row_mean == 0)
 
 // One tensor (or contiguous piece) as the kernels see it; 128 bytes so that a
 // record never straddles more cache lines than it has to.
@@ -84,6 +85,7 @@ struct LaunchArgs {
     uint32_t piece_rate;     // see sr_adamw_fast_kernel: how piece workgroups are spread over the grid
     uint32_t seed_lo, seed_hi;
     uint32_t use_ks;         // every tensor of the launch uses one DevScalars: `ks`, no table read
+    uint32_t n_rows;         // row-wise kernel: rows in the launch
     DevScalars ks;
 };
 

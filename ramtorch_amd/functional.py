@@ -80,6 +80,25 @@ class Entry:
     keep: list = field(default_factory=list)  # temporaries that must outlive the launch
 
 
+ROWWISE_MIN_LEN, ROWWISE_MAX_LEN = 512, 32768
+
+
+def rowwise_ok(e: "Entry", row_len: int, explicit_noise: bool = False) -> bool:
+    """Whether the update kernel can take the row means of this entry's gradient itself
+    (centralization, adamw.py:179-184) instead of reading them from ``row_mean``: whole tensors of
+    16-bit arrays on the GPU, 16-byte aligned, Philox noise, no debug outputs, rows a multiple of 8
+    and 512 .. 32768 elements long -- the same rule as the library's (it rejects anything else)."""
+    if explicit_noise or e.noise is not None or e.dbg is not None or e.elem_offset or e.row_mean is not None:
+        return False
+    if row_len % 8 or not (ROWWISE_MIN_LEN <= row_len <= ROWWISE_MAX_LEN) or e.p.numel() % row_len:
+        return False
+    for t in (e.p, e.g, e.m, e.v):
+        if not t.is_cuda or t.dtype not in (torch.bfloat16, torch.float16) or t.data_ptr() % 16 or not t.is_contiguous():
+            return False
+    # fp16 states come in pairs in the templated kernels; anything else is the runtime-typed kernel's
+    return (e.m.dtype == torch.float16) == (e.v.dtype == torch.float16)
+
+
 def _ptr(t: Optional[torch.Tensor]) -> int:
     return 0 if t is None else t.data_ptr()
 
@@ -124,6 +143,8 @@ def pack_descs(entries: Sequence[Entry], streamed: bool) -> np.ndarray:
         if e.row_mean is not None:
             d["row_mean"][i] = e.row_mean.data_ptr()
             d["row_len"][i] = e.row_len
+        elif e.row_len:
+            d["row_len"][i] = e.row_len   # the update kernel takes the row means itself (see rowwise_ok)
         mask = 0
         for bit, t in ((N.RT_HOST_P, e.p), (N.RT_HOST_G, e.g), (N.RT_HOST_M, e.m), (N.RT_HOST_V, e.v)):
             if not t.is_contiguous():

@@ -166,6 +166,7 @@ class AdamW(Optimizer):
         self.last_step_skipped = False    # as of the last _settle_skipped_step()
         self.fuse_in_backward = True      # the hook of make_post_accumulate_hook() is live
         self.host_arrays_ordered = False  # step_param: uploads from pinned host p / m / v wait for the current stream
+        self.fuse_row_means = True        # centralization: matrices whose rows fit a wavefront are summed inside the update
         self.max_inflight_bytes = 2 << 30  # gradients kept alive for updates still in flight (step_param)
         self.max_inflight_calls = 2       # staging chunks handed to the copy pipeline and not finished yet
         self._poll_seconds = 0.0002       # completion is read from host memory; no runtime call while waiting
@@ -199,6 +200,7 @@ class AdamW(Optimizer):
     _CONFIG_DEFAULTS = dict(chunk_size=64, optim_state_dtype=torch.bfloat16, ema_squared_dtype=None,
                             optim_state_device="cpu", seed=0, stream_chunk_bytes=256 << 20, loss_scale=1.0,
                             max_grad_norm=None, noise_source="philox", fuse_in_backward=True, host_arrays_ordered=False,
+                            fuse_row_means=True,
                             max_inflight_bytes=2 << 30, max_inflight_calls=2, _poll_seconds=0.0002,
                             gather_min_tensors=256, state_placement="auto", state_pool_min_bytes=1 << 30,
                             assume_static_layout=False)
@@ -617,10 +619,19 @@ class AdamW(Optimizer):
                     if getattr(self, "noise_source", "philox") == "reference" and inv_loss_scale == 1.0:
                         e.row_mean, e.row_len = self._row_means(g, dev, inv_loss_scale)   # torch's own mean
                     elif g.numel():
-                        # adamw.py:179-184: mean over every dim but the first (over all of them for 0-d / 1-d);
-                        # the rows of all such gradients of the step are summed in one launch below
+                        # adamw.py:179-184: mean over every dim but the first (over all of them for 0-d / 1-d)
                         rows = g.shape[0] if g.dim() >= 2 else 1
-                        cen_jobs.setdefault(dev, []).append((e, rows, g.numel() // rows if rows else 0))
+                        row_len = g.numel() // rows if rows else 0
+                        if noise is not None and p in noise:
+                            e.noise = tuple(noise[p])
+                        if debug_out is not None and p in debug_out:
+                            e.dbg = tuple(debug_out[p])
+                        if (self.__dict__.get("fuse_row_means", True) and e.p.is_cuda and e.m.is_cuda and e.v.is_cuda
+                                and F.rowwise_ok(e, row_len, explicit_noise=noise is not None)):
+                            e.row_len = row_len     # the update kernel sums the rows itself: no separate pass
+                        else:
+                            # the rows of all such gradients of the step are summed in one launch below
+                            cen_jobs.setdefault(dev, []).append((e, rows, row_len))
                 if noise is not None and p in noise:
                     e.noise = tuple(noise[p])
                 if debug_out is not None and p in debug_out:
@@ -930,8 +941,13 @@ class AdamW(Optimizer):
                 F.dtype_code(t.dtype, what)     # an unsupported dtype raises here
             if g.numel() != p.numel():
                 raise ValueError("step_param: the gradient's size differs from the parameter's")
-            if cen != 0:
-                e.row_mean, e.row_len = self._row_means(g, dev, inv_loss_scale)
+            if cen != 0 and g.numel():
+                rows = g.shape[0] if g.dim() >= 2 else 1
+                if (self.__dict__.get("fuse_row_means", True) and e.p.is_cuda and e.m.is_cuda and e.v.is_cuda
+                        and getattr(self, "noise_source", "philox") == "philox" and F.rowwise_ok(e, g.numel() // rows)):
+                    e.row_len = g.numel() // rows    # the update kernel sums the rows itself
+                else:
+                    e.row_mean, e.row_len = self._row_means(g, dev, inv_loss_scale)
             h = _handle(dev)
             state["step"] = step
             handed_over = False    # part of this tensor is already on the copy pipeline: the step counts

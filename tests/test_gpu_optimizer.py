@@ -890,6 +890,63 @@ def test_state_placement_of_two_large_optimizers_in_a_row():
         torch.cuda.empty_cache()       # tens of GiB go back to the driver: the next round starts in a used process
 
 
+@pytest.mark.parametrize("pdt,sdt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
+                                     (torch.bfloat16, torch.float16)])
+@pytest.mark.parametrize("clip", [None, 0.05])
+def test_centralization_inside_the_update_gives_the_bits_of_the_separate_row_mean_pass(pdt, sdt, clip, monkeypatch):
+    """adamw.py:179-184.  Matrices whose rows fit a wavefront (a multiple of 8, 512 .. 32768 elements) have their
+    rows summed inside the update kernel; everything else gets its means from the row-mean pass first.  Both
+    ways sum a row in the same order, so an optimizer that never sums inside the update steps to the same bits
+    (that path is checked against the oracle and the reference's op sequence elsewhere), with a loss
+    scale and with a clip coefficient on gradient and mean."""
+    shapes = [(64, 512), (7, 4096), (3, 14336), (5, 520), (3, 32768), (2, 3, 256), (40, 504), (9, 1000), (4, 516),
+              (4096,), (3, 32776), (1, 512), (300, 8)]
+    eligible = {0, 1, 2, 3, 4, 5, 7, 9, 11}   # rows a multiple of 8 and 512 .. 32768 long ((2,3,256): rows of 768)
+    from ramtorch_amd import functional as F
+    passes = []
+    real = F.row_means_multi
+    monkeypatch.setattr(F, "row_means_multi", lambda h, jobs, *a, **k: (passes.append(len(jobs)), real(h, jobs, *a, **k))[1])
+
+    def make(**attrs):
+        ps, grads = _make_params(shapes, 9100)
+        ps = [torch.nn.Parameter(p.detach().to(pdt)) for p in ps]
+        opt = ramtorch_amd.AdamW(ps, lr=2e-3, centralization=0.7, storage_device="cuda", dtype=sdt, seed=5,
+                                 loss_scale=8.0, max_grad_norm=clip)
+        for k, v in attrs.items():
+            setattr(opt, k, v)
+        return ps, grads, opt
+
+    ps_a, grads, a = make()
+    ps_b, _, b = make(fuse_row_means=False)
+    for step in range(3):
+        for x, y, g in zip(ps_a, ps_b, grads):
+            x.grad = (g.float() * (8.0 + step)).to(pdt).cuda()
+            y.grad = x.grad.clone()
+        passes.clear()
+        a.step()
+        assert passes == [len(shapes) - len(eligible)], passes     # the rest is summed inside the update
+        passes.clear()
+        b.step()
+        assert passes == [len(shapes)]
+        torch.cuda.synchronize()
+        for i, (x, y) in enumerate(zip(ps_a, ps_b)):
+            assert nmis(x.detach(), y.detach()) == 0, (step, shapes[i])
+            assert nmis(a.state[x]["ema"], b.state[y]["ema"]) == 0, (step, shapes[i])
+            assert nmis(a.state[x]["ema_squared"], b.state[y]["ema_squared"]) == 0, (step, shapes[i])
+    assert not a.step_was_skipped() and not b.step_was_skipped()
+    if clip is None:
+        # single parameters handed over as a backward hook would: the same choice per tensor
+        for opt, ps in ((a, ps_a), (b, ps_b)):
+            for i in (1, 6, 2):
+                opt.step_param(ps[i])
+            opt.step()
+        torch.cuda.synchronize()
+        for i, (x, y) in enumerate(zip(ps_a, ps_b)):
+            assert nmis(x.detach(), y.detach()) == 0, shapes[i]
+            assert nmis(a.state[x]["ema_squared"], b.state[y]["ema_squared"]) == 0, shapes[i]
+            assert a.state[x]["step"] == b.state[y]["step"] == 4
+
+
 def test_frozen_layout_steps_like_the_full_path_and_notices_moved_gradients():
     """assume_static_layout: after the first step the optimizer only checks that parameters and
     gradients are where they were.  Same bits as an optimizer that gathers everything every step,
