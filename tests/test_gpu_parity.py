@@ -411,6 +411,21 @@ def test_bad_arguments_are_rejected(handle):
     e.tensor_id = 1 << 30
     with pytest.raises(N.NativeError, match="tensor_id"):
         F.step_resident(handle, [e], [F.make_scalars(step=1, **HP0)], seed=0, explicit_noise=False)
+    # centralization without row means: only for tensors the row-wise kernel takes (rows a multiple of 8, 512 .. 32768)
+    e.tensor_id = 0
+    cen = [F.make_scalars(step=1, centralization=0.5, **HP0)]
+    with pytest.raises(N.NativeError, match="row_len"):
+        F.step_resident(handle, [e], cen, seed=0, explicit_noise=False)
+    e.row_len = 16
+    with pytest.raises(N.NativeError, match="without row_mean"):
+        F.step_resident(handle, [e], cen, seed=0, explicit_noise=False)
+    big = torch.zeros(1024, dtype=torch.bfloat16, device="cuda")
+    e2 = F.Entry(p=big, g=big.clone(), m=big.clone(), v=big.clone(), step=1, scalars_idx=0, tensor_id=0, row_len=520)
+    with pytest.raises(N.NativeError, match="without row_mean"):     # 1024 is not a multiple of 520
+        F.step_resident(handle, [e2], cen, seed=0, explicit_noise=False)
+    e2.row_len = 512
+    F.step_resident(handle, [e2], cen, seed=0, explicit_noise=False)   # two rows of 512: taken
+    torch.cuda.synchronize()
 
 
 def test_kernel_timing_history(handle):
