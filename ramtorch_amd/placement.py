@@ -129,12 +129,24 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
         report.update(placed=placed, filler_GiB=held_bytes / GIB, same_GBps=same, cross_GBps=cross)
         return t
 
+    def out_of_time(next_cost=0.0):
+        # (allocations take their time while the driver is still clearing memory that was released
+        # shortly before: a block of 16 GiB up to half a second)
+        if time.monotonic() - t0 + next_cost > max_seconds:
+            report["reason"] = f"no place showed the whole gain within {max_seconds:g} s"
+            return True
+        return False
+
+    try_cost = 0.0   # what the last try took, the allocation of its block included
     try:
         while b is None:
             free, _ = torch.cuda.mem_get_info(device)
             if bytes_b + 2 * GIB > free:
                 report["reason"] = "not enough free device memory to try another place"
                 break
+            if report["tries"] and out_of_time(try_cost):
+                break
+            t_try = time.monotonic()
             try:
                 cand = handle.dev_hold(bytes_b)   # the place the second pool would get right now
             except N.NativeError:
@@ -146,6 +158,7 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
                 report["reason"] = "pools too small for the probe to tell places apart"
                 break
             same, cross, full = summary(res)
+            try_cost = time.monotonic() - t_try
             report["tries"] += 1
             if report["cross_GBps"] is None:
                 report.update(same_GBps=same, cross_GBps=cross)
@@ -166,8 +179,7 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
             else:
                 handle.dev_release(cand)
             free, _ = torch.cuda.mem_get_info(device)
-            if time.monotonic() - t0 > max_seconds:
-                report["reason"] = f"no place showed the whole gain within {max_seconds:g} s"
+            if out_of_time():
                 break
             if held_bytes + step_bytes > budget or step_bytes + bytes_b + 4 * GIB > free:
                 report["reason"] = (f"no place showed the whole gain with {held_bytes / GIB:.0f} GiB occupied "
@@ -177,8 +189,12 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
                 for _ in range(max(1, step_bytes // filler_bytes)):
                     held.append(handle.dev_hold(filler_bytes))
                     held_bytes += filler_bytes
+                    if out_of_time():
+                        break
             except N.NativeError:
                 report["reason"] = "not enough free device memory to occupy more"
+                break
+            if report["reason"]:
                 break
         if b is None and best is not None and best[2] >= 1.01 * best[1]:
             report["reason"] = (report["reason"] or "") + "; the best place seen was taken"
