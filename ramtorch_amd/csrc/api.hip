@@ -140,7 +140,9 @@ struct Batch {            // tensors of one dtype combination inside a table ima
     uint32_t first_piece, n_pieces;            // pieces served by the fast kernel's first workgroups
     uint32_t first_generic, n_generic;         // chunk range of the generic kernel
     uint32_t first_cen_range, n_cen_ranges, n_cen_units;  // the same lists for tensors with centralization
-    uint32_t first_rw_range, n_rw_ranges, n_rw_rows;      // tensors whose row means the kernel takes itself: first rows
+    // tensors whose row means the kernel takes itself, as lists of first rows: [0] rows longer than
+    // kRowwiseShortMax elements, [1] the others
+    uint32_t first_rw_range[2], n_rw_ranges[2], n_rw_rows[2];
 };
 
 struct Plan {
@@ -252,6 +254,7 @@ struct KernelPair {
     MultiKernel generic;  // unaligned tensors, debug outputs, leftovers without a piece path, rows shorter than 8
     MultiKernel fast_cen; // whole fast units of aligned tensors with centralization (16-bit layouts, Philox), or NULL
     MultiKernel rowwise;  // whole tensors with centralization whose row means the kernel takes itself (same layouts), or NULL
+    MultiKernel rowwise_short;  // the same for rows of at most kRowwiseShortMax elements
 };
 
 template <int P, int G, int M, int V>
@@ -261,15 +264,16 @@ static KernelPair pick_noise(int noise) {
     if constexpr (wide) {
         if (noise == RT_NOISE_EXPLICIT)
             return {sr_adamw_fast_wide_kernel<P, G, M, V, RT_NOISE_EXPLICIT>,
-                    sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_EXPLICIT>, nullptr, nullptr};
+                    sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_EXPLICIT>, nullptr, nullptr, nullptr};
         return {sr_adamw_fast_wide_kernel<P, G, M, V, RT_NOISE_PHILOX>,
-                sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_PHILOX>, nullptr, nullptr};
+                sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_PHILOX>, nullptr, nullptr, nullptr};
     } else {
         if (noise == RT_NOISE_EXPLICIT)
             return {sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_EXPLICIT>,
-                    sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_EXPLICIT>, nullptr, nullptr};
+                    sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_EXPLICIT>, nullptr, nullptr, nullptr};
         return {sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_PHILOX>, sr_adamw_generic_kernel<P, G, M, V, RT_NOISE_PHILOX>,
-                sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_PHILOX, true>, sr_adamw_rowwise_kernel<P, G, M, V>};
+                sr_adamw_fast_kernel<P, G, M, V, RT_NOISE_PHILOX, true>, sr_adamw_rowwise_kernel<P, G, M, V, false>,
+                sr_adamw_rowwise_kernel<P, G, M, V, true>};
     }
 }
 // State dtype pairs the templated kernels are instantiated for: every bf16 / fp32 mix, and both fp16.
@@ -508,17 +512,19 @@ static void build_image(rt_handle* h, const rt_tensor_desc* descs, uint32_t n, c
         b.n_cen_ranges = (uint32_t)ranges.size() - b.first_cen_range;
         b.n_cen_units = cen_units;
         // Tensors whose row means the update takes itself: whole tensors, a wavefront per row.
-        b.first_rw_range = (uint32_t)ranges.size();
-        uint64_t rw_rows = 0;
-        for (size_t k = k0; k < k1; ++k) {
-            const DevTensor& t = tens[k];
-            if (!(t.flags & kFlagRowwise)) continue;
-            ranges.push_back((uint32_t)rw_rows);
-            fast_tens.push_back(t);
-            rw_rows += t.numel / t.row_len;
+        for (int kind = 0; kind < 2; ++kind) {
+            b.first_rw_range[kind] = (uint32_t)ranges.size();
+            uint64_t rw_rows = 0;
+            for (size_t k = k0; k < k1; ++k) {
+                const DevTensor& t = tens[k];
+                if (!(t.flags & kFlagRowwise) || (int)(t.row_len <= kRowwiseShortMax) != kind) continue;
+                ranges.push_back((uint32_t)rw_rows);
+                fast_tens.push_back(t);
+                rw_rows += t.numel / t.row_len;
+            }
+            b.n_rw_ranges[kind] = (uint32_t)ranges.size() - b.first_rw_range[kind];
+            b.n_rw_rows[kind] = (uint32_t)std::min<uint64_t>(rw_rows, 0xFFFFFFFFull);   // checked against the grid limit at launch
         }
-        b.n_rw_ranges = (uint32_t)ranges.size() - b.first_rw_range;
-        b.n_rw_rows = (uint32_t)std::min<uint64_t>(rw_rows, 0xFFFFFFFFull);   // checked against the grid limit at launch
         b.first_generic = (uint32_t)chunks.size();
         for (size_t k = k0; k < k1; ++k) {
             const DevTensor& t = tens[k];
@@ -659,18 +665,20 @@ static int enqueue_kernels(const Plan& plan, const uint8_t* base, uint64_t seed,
             c.n_pieces = c.n_piece_wgs = c.piece_rate = 0;
             launches.push_back(Launch{k.fast_cen, b.n_cen_units, c});
         }
-        if (b.n_rw_rows) {
-            if (!k.rowwise) return fail(RT_EHIP, "internal: row-wise tensors without a kernel for them");
-            const uint64_t rw_grid = ((uint64_t)b.n_rw_rows + kThreads / 64 - 1) / (kThreads / 64);
-            if (b.n_rw_rows == 0xFFFFFFFFu || rw_grid > kMaxGrid)
+        for (int kind = 0; kind < 2; ++kind) {
+            if (!b.n_rw_rows[kind]) continue;
+            const MultiKernel kern = kind ? k.rowwise_short : k.rowwise;
+            if (!kern) return fail(RT_EHIP, "internal: row-wise tensors without a kernel for them");
+            const uint64_t rw_grid = ((uint64_t)b.n_rw_rows[kind] + kThreads / 64 - 1) / (kThreads / 64);
+            if (b.n_rw_rows[kind] == 0xFFFFFFFFu || rw_grid > kMaxGrid)
                 return fail(RT_EUNSUPPORTED, "too many rows in one launch");
             LaunchArgs c = a;
-            c.first = (const uint32_t*)(base + plan.off_ranges) + b.first_rw_range;
-            c.fast_tensors = (const DevTensor*)(base + plan.off_fast_tensors) + b.first_rw_range;
-            c.n_ranges = b.n_rw_ranges;
-            c.n_rows = b.n_rw_rows;
+            c.first = (const uint32_t*)(base + plan.off_ranges) + b.first_rw_range[kind];
+            c.fast_tensors = (const DevTensor*)(base + plan.off_fast_tensors) + b.first_rw_range[kind];
+            c.n_ranges = b.n_rw_ranges[kind];
+            c.n_rows = b.n_rw_rows[kind];
             c.n_pieces = c.n_piece_wgs = c.piece_rate = 0;
-            launches.push_back(Launch{k.rowwise, (uint32_t)rw_grid, c});
+            launches.push_back(Launch{kern, (uint32_t)rw_grid, c});
         }
     }
     for (size_t i = 0; i < launches.size(); ++i) {
