@@ -80,7 +80,7 @@ OFFLINE_TRAFFIC = {
     "mixed": (160_597_606_615, _TRAFFIC_FILE),      # the update launch; its norm pass fetches 32 120 545 889 B more
     "small": (1_090_935_301, _TRAFFIC_FILE),
     "cfg0": (335_774_529, _TRAFFIC_FILE),
-    "central": (116_177_807_872, _TRAFFIC_FILE),   # row-wise kernel with one instance for all rows: every gradient row read twice, 77 % of the second reads out of the L2
+    "central": (116_001_647_514, _TRAFFIC_FILE),   # row-wise kernels: the rows of 14 336 elements are read twice, the second time mostly from HBM
     "any": (8_292_259_533, _TRAFFIC_FILE),
 }
 HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
