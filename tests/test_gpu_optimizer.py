@@ -947,6 +947,55 @@ def test_centralization_inside_the_update_gives_the_bits_of_the_separate_row_mea
             assert a.state[x]["step"] == b.state[y]["step"] == 4
 
 
+def test_random_sets_step_alike_with_row_sums_inside_the_update_and_in_a_pass_of_their_own():
+    """Seeded random parameter sets -- row lengths on both sides of every limit of the row-wise kernel
+    (8, 512, 4096, 32768), 1-D to 3-D shapes, bf16 / fp16 parameters, bf16 / fp16 / fp32 states, two groups
+    with different centralization (0 included), loss scale, clip, gradients that are missing in some
+    steps: an optimizer that sums rows inside the update and one that never does agree bit for bit."""
+    lens = [8, 64, 504, 512, 520, 1000, 1024, 4088, 4096, 4104, 8192, 14336, 32768, 32776, 516, 3, 40000]
+    for seed in range(40):
+        rng = np.random.default_rng(seed)
+        shapes = []
+        for _ in range(int(rng.integers(3, 14))):
+            L = int(rng.choice(lens))
+            rows = int(rng.integers(1, max(2, min(40, 400000 // L))))
+            kind = rng.integers(0, 4)
+            shapes.append((L,) if kind == 0 else (rows, 4, L // 4) if kind == 1 and L % 4 == 0 else (rows, L))
+        pdt = [torch.bfloat16, torch.float16][int(rng.integers(0, 2))]
+        sdt = [torch.bfloat16, torch.float16, torch.float32][int(rng.integers(0, 3))]
+        clip = None if rng.random() < 0.5 else float(rng.choice([0.01, 1.0, 100.0]))
+        ls = float(rng.choice([1.0, 8.0, 1024.0]))
+        cut = int(rng.integers(1, len(shapes)))
+        cens = (float(rng.choice([0.0, 0.3, 1.0])), float(rng.choice([0.5, 1.0])))
+
+        def make(fuse):
+            ps, grads = _make_params(shapes, 1000 + seed)
+            ps = [torch.nn.Parameter(p.detach().to(pdt)) for p in ps]
+            opt = ramtorch_amd.AdamW([{"params": ps[:cut], "centralization": cens[0]},
+                                      {"params": ps[cut:], "centralization": cens[1], "lr": 3e-3}],
+                                     lr=1e-3, storage_device="cuda", dtype=sdt, seed=seed, loss_scale=ls, max_grad_norm=clip)
+            opt.fuse_row_means = fuse
+            return ps, grads, opt
+
+        ps_a, grads, a = make(True)
+        ps_b, _, b = make(False)
+        for step in range(3):
+            for x, y, g in zip(ps_a, ps_b, grads):
+                if rng.random() < 0.15:
+                    x.grad = y.grad = None
+                    continue
+                x.grad = (g.float() * (ls * (1.0 + step))).to(pdt).cuda()
+                y.grad = x.grad.clone()
+            a.step(); b.step()
+            torch.cuda.synchronize()
+            for i, (x, y) in enumerate(zip(ps_a, ps_b)):
+                what = (seed, step, shapes[i], pdt, sdt)
+                assert nmis(x.detach(), y.detach()) == 0, what
+                assert nmis(a.state[x]["ema"], b.state[y]["ema"]) == 0, what
+                assert nmis(a.state[x]["ema_squared"], b.state[y]["ema_squared"]) == 0, what
+                assert a.state[x]["step"] == b.state[y]["step"], what
+
+
 def test_frozen_layout_steps_like_the_full_path_and_notices_moved_gradients():
     """assume_static_layout: after the first step the optimizer only checks that parameters and
     gradients are where they were.  Same bits as an optimizer that gathers everything every step,
