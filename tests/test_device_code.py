@@ -63,3 +63,11 @@ def test_update_kernels_keep_their_occupancy(device_asm):
         assert m, "kernel metadata not found"
         print(cen, "vgpr_count", m.group(2))
         assert int(m.group(2)) <= limit, m.group(2)
+    # the row-wise centralizing kernel: four waves per SIMD for rows that are read twice, three for the
+    # instance that keeps a row's gradient in registers
+    for short, limit in (("Lb0", 128), ("Lb1", 168)):
+        m = re.search(r"\.name:\s+(_ZN2rt23sr_adamw_rowwise_kernelILi0ELi0ELi0ELi0E" + short +
+                      r"EE\w+)\n(?:.*\n)*?\s+\.vgpr_count:\s+(\d+)", device_asm)
+        assert m, "kernel metadata not found"
+        print("row-wise", short, "vgpr_count", m.group(2))
+        assert int(m.group(2)) <= limit, m.group(2)
