@@ -74,7 +74,7 @@ class _HeldBlock:
 def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: int, *,
                min_gain: float = 1.05, min_gain_anywhere: float = 1.02, filler_bytes: int = 2 * GIB,
                step_bytes: int = 16 * GIB, max_filler_bytes: int = 112 * GIB, max_fraction_of_free: float = 0.5,
-               max_seconds: float = 1.2, log: Optional[Callable[[str], None]] = None):
+               max_seconds: float = 1.0, log: Optional[Callable[[str], None]] = None):
     """Two zeroed byte pools on ``device`` such that arrays in the second are, as far as it can be
     arranged, in another HBM region than the corresponding arrays in the first.  Returns
     (pool_a, pool_b, report).
