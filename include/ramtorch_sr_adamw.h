@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define RT_ABI_VERSION 3
+#define RT_ABI_VERSION 4
 
 /* error codes */
 #define RT_OK 0
@@ -360,6 +360,46 @@ int rt_host_link_probe(rt_handle* h, uint64_t bytes, int reps, double out[3]);
  */
 int rt_dev_hold(rt_handle* h, uint64_t bytes, void** out);
 int rt_dev_release(rt_handle* h, void* p);
+
+/*
+ * Two zeroed device blocks of at least bytes_a and bytes_b for arrays that an
+ * update reads and writes together (the optimizer's ema and ema_squared pools),
+ * placed so that the two never share an HBM region (see rt_stream_probe): *a
+ * and *b.  Nothing in the reference corresponds to it.  The blocks are built
+ * from physical chunks of 1 GiB taken one by one through the virtual-memory
+ * API (hipMemCreate), each probed with the update's traffic -- p, g, ema in the
+ * first chunk, ema_squared at the chunk's two ends -- and sorted into "with the
+ * first chunk" and "elsewhere"; one block is mapped from chunks of the first
+ * kind, the other from chunks of the second, side by side in an address range
+ * of its own.  Chunk by chunk, so it works as well in a process whose earlier
+ * allocations have left the free memory in scattered order, where one large
+ * allocation straddles regions.  On the way the search holds at most
+ * max_extra_bytes more than the two blocks and gives up after max_seconds;
+ * blocks it could not complete from the right kind of chunk are completed with
+ * others.  Each block is given back with rt_dev_release (which waits for the
+ * device first).  RT_EUNSUPPORTED when the runtime has no such allocations.
+ * ref_p, ref_m, ref_v, ref_elems (optional, ref_elems == 0: none): three
+ * disjoint 16-byte-aligned arrays of ref_elems 16-bit elements in the memory
+ * of the parameters the blocks will be used with (ref_elems a multiple of
+ * 8192 between 2^25 and 2^27).  The probes then run with the first two as p
+ * and ema, and the third as ema_squared gives the rate of the parameters' own
+ * region, so that the kinds are "with the parameters" (no faster than that)
+ * and "elsewhere" (3.5 % faster at least): *a is built from
+ * the first kind (or, when that region has too few free chunks, from the
+ * second as well), *b from the second, and an update never has p, ema and
+ * ema_squared in one region nor, with *a complete, in three.  The probe
+ * writes the reference arrays back bit for bit as they are (it stores p ^ g
+ * with g zero); nothing else may write them while the call runs.
+ *   report[0] = 1 when both blocks are wholly of their kind, else 0
+ *   report[1] = share of the second block that lies apart from the first
+ *   report[2] = chunks taken and probed       report[3] = seconds
+ *   report[4], report[5] = GB/s of the probe within one region / across two
+ *   report[6] = why the search ended: 0 complete, 1 memory limit, 2 time limit, 3 no free chunk left
+ *   report[7] = 1 when *a is the block in the first chunk's region
+ */
+int rt_dev_hold_pair(rt_handle* h, uint64_t bytes_a, uint64_t bytes_b, uint64_t max_extra_bytes, double max_seconds,
+                     void* ref_p, void* ref_m, void* ref_v, uint64_t ref_elems, void** a, void** b,
+                     double report[8], void* stream);
 
 /*
  * Self-test, nothing in the reference corresponds to it.  The update kernels

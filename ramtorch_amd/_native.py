@@ -15,7 +15,7 @@ import weakref
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "_lib", "libramtorch_sr_adamw.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 RT_OK = 0
 RT_EINVAL, RT_EHIP, RT_ENOMEM, RT_EUNSUPPORTED = -1, -2, -3, -4
@@ -30,7 +30,7 @@ EXPORTS = (
     "rt_grad_norm", "rt_row_means", "rt_sr_copy", "rt_set_timing", "rt_last_kernel_ms", "rt_kernel_ms_history", "rt_streamed_stats",
     "rt_stream_probe", "rt_streamed_timeline", "rt_streamed_plan",
     "rt_step_streamed_async", "rt_streamed_wait", "rt_streamed_completed",
-    "rt_grad_norm_static", "rt_host_link_probe", "rt_selftest_sqrt", "rt_dev_hold", "rt_dev_release",
+    "rt_grad_norm_static", "rt_host_link_probe", "rt_selftest_sqrt", "rt_dev_hold", "rt_dev_release", "rt_dev_hold_pair",
     "rt_streamed_bounce_stats", "rt_row_means_multi", "rt_streamed_schedule",
 )
 
@@ -148,6 +148,9 @@ def lib() -> ctypes.CDLL:
     L.rt_dev_hold.argtypes = [vp, u64, ctypes.POINTER(vp)]
     L.rt_dev_release.restype = i32
     L.rt_dev_release.argtypes = [vp, vp]
+    L.rt_dev_hold_pair.restype = i32
+    L.rt_dev_hold_pair.argtypes = [vp, u64, u64, u64, ctypes.c_double, vp, vp, vp, u64, ctypes.POINTER(vp),
+                                   ctypes.POINTER(vp), ctypes.POINTER(ctypes.c_double), vp]
     L.rt_selftest_sqrt.restype = i32
     L.rt_selftest_sqrt.argtypes = [vp, ctypes.POINTER(u64)]
     L.rt_row_means_multi.restype = i32
@@ -279,6 +282,17 @@ class Handle:
         with self._lock:
             check(lib().rt_dev_hold(self.ptr, int(nbytes), ctypes.byref(out)))
         return out.value
+
+    def dev_hold_pair(self, bytes_a: int, bytes_b: int, max_extra_bytes: int, max_seconds: float, ref=None, stream=0):
+        """(address a, address b, report) of two zeroed blocks that never share an HBM region (see
+        rt_dev_hold_pair); ``ref``: optional (address, address, address, elements) of three arrays in parameter memory."""
+        a, b = ctypes.c_void_p(), ctypes.c_void_p()
+        rep = (ctypes.c_double * 8)()
+        rp, rm, rv, rn = ref if ref else (None, None, None, 0)
+        with self._lock:
+            check(lib().rt_dev_hold_pair(self.ptr, int(bytes_a), int(bytes_b), int(max_extra_bytes), float(max_seconds),
+                                         rp, rm, rv, int(rn), ctypes.byref(a), ctypes.byref(b), rep, stream))
+        return a.value, b.value, list(rep)
 
     def dev_release(self, addr: int) -> None:
         with self._lock:

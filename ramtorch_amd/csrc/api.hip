@@ -1948,8 +1948,321 @@ int rt_dev_hold(rt_handle* h, uint64_t bytes, void** out) {
     return RT_OK;
 }
 
+// ---------------------------------------------------------------------------
+// rt_dev_hold_pair: two blocks assembled from physical chunks that were probed one by one.
+// ---------------------------------------------------------------------------
+namespace {
+constexpr size_t kPairChunk = 1ull << 30;          // physical chunks of 1 GiB
+constexpr uint64_t kPairProbeElems = 128ull << 20;  // 256 MiB of bf16 per probed array: three of them and a fourth fit a chunk
+constexpr uint64_t kPairMinProbeElems = 32ull << 20;  // shorter probes scatter too much to tell the regions apart
+
+struct PairBlock {   // one block handed out by rt_dev_hold_pair
+    size_t bytes = 0;
+    int device = 0;
+    std::vector<hipMemGenericAllocationHandle_t> chunks;
+};
+std::mutex g_pair_mutex;
+std::map<void*, PairBlock> g_pair_blocks;
+
+// Unmaps `mapped` chunks of 1 GiB that sit side by side from `va` on, releases their handles and
+// frees the address range of `reserved` bytes; goes on after an error and returns the first one.
+static hipError_t pair_teardown(void* va, size_t reserved, std::vector<hipMemGenericAllocationHandle_t>& chunks,
+                                size_t mapped) {
+    hipError_t first = hipSuccess;
+    auto note = [&](hipError_t e) { if (e != hipSuccess && first == hipSuccess) first = e; };
+    for (size_t i = 0; va && i < mapped; ++i) note(hipMemUnmap((uint8_t*)va + i * kPairChunk, kPairChunk));
+    for (auto hnd : chunks) note(hipMemRelease(hnd));
+    chunks.clear();
+    if (va && reserved) note(hipMemAddressFree(va, reserved));
+    return first;
+}
+}  // namespace
+
+int rt_dev_hold_pair(rt_handle* h, uint64_t bytes_a, uint64_t bytes_b, uint64_t max_extra_bytes, double max_seconds,
+                     void* ref_p, void* ref_m, void* ref_v, uint64_t ref_elems, void** a_out, void** b_out,
+                     double report[8], void* stream_) {
+    if (!h || !a_out || !b_out || !report) return fail(RT_EINVAL, "NULL argument");
+    *a_out = *b_out = nullptr;
+    for (int i = 0; i < 8; ++i) report[i] = 0.0;
+    if (bytes_a == 0 || bytes_b == 0) return fail(RT_EINVAL, "sizes must be positive");
+    const bool has_ref = ref_elems != 0;
+    if (has_ref) {
+        if (!ref_p || !ref_m || !ref_v || (((uintptr_t)ref_p | (uintptr_t)ref_m | (uintptr_t)ref_v) & 15u) != 0)
+            return fail(RT_EINVAL, "reference arrays must be 16-byte aligned device addresses");
+        if (ref_elems % kChunkElems != 0 || ref_elems < kPairMinProbeElems || ref_elems > kPairProbeElems)
+            return fail(RT_EINVAL, "ref_elems must be a multiple of %u between %llu and %llu", kChunkElems,
+                        (unsigned long long)kPairMinProbeElems, (unsigned long long)kPairProbeElems);
+    }
+    const uint64_t probe_elems = has_ref ? ref_elems : kPairProbeElems;
+    HIP_TRY(hipSetDevice(h->device));
+    hipStream_t stream = (hipStream_t)stream_;
+    const auto t_start = std::chrono::steady_clock::now();
+    auto elapsed = [&] { return std::chrono::duration<double>(std::chrono::steady_clock::now() - t_start).count(); };
+    const size_t C = kPairChunk;
+    const size_t n_a = (bytes_a + C - 1) / C, n_b = (bytes_b + C - 1) / C;
+    const size_t n_max = n_a + n_b + (size_t)(max_extra_bytes / C);
+
+    hipMemAllocationProp prop;
+    memset(&prop, 0, sizeof(prop));
+    prop.type = hipMemAllocationTypePinned;
+    prop.location.type = hipMemLocationTypeDevice;
+    prop.location.id = h->device;
+    hipMemAccessDesc access;
+    memset(&access, 0, sizeof(access));
+    access.location = prop.location;
+    access.flags = hipMemAccessFlagsProtReadWrite;
+    size_t gran = 0;
+    if (hipMemGetAllocationGranularity(&gran, &prop, hipMemAllocationGranularityRecommended) != hipSuccess || gran == 0 ||
+        C % gran != 0) {
+        (void)hipGetLastError();
+        return fail(RT_EUNSUPPORTED, "the device has no virtual-memory allocation of 1 GiB chunks");
+    }
+
+    // Every chunk is mapped where it was taken, side by side in one scratch range, and probed there.
+    void* scratch = nullptr;
+    if (hipMemAddressReserve(&scratch, n_max * C, 0, nullptr, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(RT_EUNSUPPORTED, "reserving %zu GiB of device address space failed", n_max);
+    }
+    std::vector<hipMemGenericAllocationHandle_t> chunks;   // chunk k is mapped at scratch + k * C
+    std::vector<float> rate;                                // GB/s of the probe with ema_squared in chunk k; < 0: mixed
+    auto fail_all = [&](int code, const char* what, hipError_t e) {
+        (void)hipDeviceSynchronize();
+        (void)pair_teardown(scratch, n_max * C, chunks, chunks.size());
+        (void)hipGetLastError();
+        return fail(code, "%s: %s", what, hipGetErrorString(e));
+    };
+    // The update's traffic with ema_squared where the caller says.  Without reference arrays p, g and ema
+    // stand in the first chunk.  With them, p and ema are the caller's own arrays -- parameter memory, so
+    // that "the first kind" means "where the parameters are"; the probe writes p ^ g and ema ^ g back and
+    // g is a zeroed part of the first chunk, so every bit of them stays as it is.
+    auto probe = [&](void* v, float* gbps) -> hipError_t {
+        uint8_t* base = (uint8_t*)scratch;
+        const size_t arr = probe_elems * 2;
+        const uint64_t pp = has_ref ? (uint64_t)ref_p : (uint64_t)base;
+        const uint64_t gg = has_ref ? (uint64_t)base : (uint64_t)(base + arr);
+        const uint64_t mm = has_ref ? (uint64_t)ref_m : (uint64_t)(base + 2 * arr);
+        const dim3 grid((uint32_t)(probe_elems / kChunkElems));
+        hipLaunchKernelGGL(stream_probe_kernel, grid, dim3(kThreads), 0, stream, pp, gg, mm, (uint64_t)v);
+        hipError_t e = hipEventRecord(h->t0, stream);
+        for (int r = 0; r < 3 && e == hipSuccess; ++r)
+            hipLaunchKernelGGL(stream_probe_kernel, grid, dim3(kThreads), 0, stream, pp, gg, mm, (uint64_t)v);
+        if (e == hipSuccess) e = hipGetLastError();
+        if (e == hipSuccess) e = hipEventRecord(h->t1, stream);
+        if (e == hipSuccess) e = hipEventSynchronize(h->t1);
+        float ms = 0.0f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, h->t0, h->t1);
+        if (e == hipSuccess) *gbps = (float)(14.0 * (double)probe_elems * 3 / (ms * 1e-3) / 1e9);
+        return e;
+    };
+
+    float lo = 0.0f, hi = 0.0f;   // mean rates of the two kinds of chunk
+    size_t near_n = 0, far_n = 0;
+    // Two kinds of chunk: those that run at the rate of the first chunk's own region and those that run at the
+    // higher rate of another region.  Two-means over the rates seen so far; the kinds count as told apart only
+    // when their means differ by 4 % (single probes scatter by 2 - 3 %, the regions differ by 7 %).
+    float ref_level = 0.0f;   // with reference arrays: the rate with ema_squared in parameter memory as well
+    auto classify = [&]() -> float {
+        near_n = far_n = 0;
+        float mn = 1e30f, mx = 0.0f;
+        for (float r : rate)
+            if (r >= 0.0f) { mn = std::min(mn, r); mx = std::max(mx, r); }
+        if (mx == 0.0f) return 1e30f;
+        float c1 = mn, c2 = mx;
+        for (int it = 0; it < 8; ++it) {
+            const float mid = 0.5f * (c1 + c2);
+            double s1 = 0, s2 = 0;
+            size_t k1 = 0, k2 = 0;
+            for (float r : rate) {
+                if (r < 0.0f) continue;
+                if (r < mid) { s1 += r; ++k1; } else { s2 += r; ++k2; }
+            }
+            if (k1) c1 = (float)(s1 / k1);
+            if (k2) c2 = (float)(s2 / k2);
+        }
+        lo = c1;
+        hi = c2;
+        // One kind only so far: without reference arrays it is the first chunk's; with them it is "elsewhere"
+        // when it runs 3.5 % faster than the probe that has all its arrays inside the parameters' memory.
+        float thr = 1e30f;
+        if (c2 >= 1.04f * c1) thr = 0.5f * (c1 + c2);
+        else if (has_ref && 0.5f * (c1 + c2) >= 1.035f * ref_level) thr = 0.0f;
+        for (float r : rate) {
+            if (r < 0.0f) continue;
+            (r < thr ? near_n : far_n) += 1;
+        }
+        return thr;
+    };
+    // Without reference arrays either block may be the one in the first chunk's region.  With them, the second
+    // block is the one away from the parameters and the first lies with them; when their region has too few free
+    // chunks for that, the search runs to its limits and the first block is completed with chunks from elsewhere
+    // (the parameters then have their region to themselves, which is still better than sharing it with both).
+    auto is_complete = [&] {
+        if (has_ref) return far_n >= n_b && near_n >= n_a;
+        return (near_n >= n_a && far_n >= n_b) || (far_n >= n_a && near_n >= n_b);
+    };
+    int ended = 0;   // 0: both blocks complete, 1: memory limit, 2: time limit, 3: no more free chunks
+    bool complete = false;
+    while (true) {
+        classify();
+        if (is_complete()) {
+            complete = true;
+            break;
+        }
+        if (chunks.size() >= n_max) { ended = 1; break; }
+        if (!chunks.empty() && elapsed() > max_seconds) { ended = 2; break; }
+        hipMemGenericAllocationHandle_t hnd;
+        hipError_t e = hipMemCreate(&hnd, C, &prop, 0);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            ended = 3;
+            break;
+        }
+        uint8_t* at = (uint8_t*)scratch + chunks.size() * C;
+        e = hipMemMap(at, C, 0, hnd, 0);
+        if (e != hipSuccess) {
+            (void)hipMemRelease(hnd);
+            return fail_all(RT_EHIP, "hipMemMap", e);
+        }
+        chunks.push_back(hnd);
+        e = hipMemSetAccess(at, C, &access, 1);
+        if (e != hipSuccess) return fail_all(RT_EHIP, "hipMemSetAccess", e);
+        float r0 = 0.0f, r1 = 0.0f;
+        const size_t arr = probe_elems * 2;
+        if (chunks.size() == 1 && has_ref) {
+            // the first chunk holds the zeroed stand-in for the gradient at its beginning
+            e = hipMemsetAsync(at, 0, arr, stream);
+            float l0 = 0.0f, l1 = 0.0f;
+            if (e == hipSuccess) e = probe(ref_v, &l0);
+            if (e == hipSuccess) e = probe(ref_v, &l1);
+            ref_level = std::max(l0, l1);
+            if (e == hipSuccess) e = probe(at + arr, &r0);
+            if (e == hipSuccess) e = probe(at + C - arr, &r1);
+        } else if (chunks.size() == 1) {
+            // all four arrays inside the first chunk: the rate of one region
+            e = probe(at + 3 * arr, &r0);
+            r1 = r0;
+        } else {
+            e = probe(at, &r0);
+            if (e == hipSuccess) e = probe(at + C - arr, &r1);
+        }
+        if (e != hipSuccess) return fail_all(RT_EHIP, "probing a chunk", e);
+        const float mean = 0.5f * (r0 + r1);
+        // a chunk whose two ends disagree lies across a region boundary: it serves neither block
+        rate.push_back(fabsf(r0 - r1) > 0.04f * mean ? -1.0f : mean);
+    }
+    const float thr = classify();
+    complete = is_complete();
+    // Without reference arrays: the block that must lie in one region takes the chunks of the first chunk's kind
+    // ("near"), the other takes chunks that are anywhere else -- whichever way round the counts allow.
+    const bool a_is_near = has_ref ? true : !(complete && !(near_n >= n_a && far_n >= n_b));
+    std::vector<size_t> pick_a, pick_b, rest;
+    for (size_t k = 0; k < chunks.size(); ++k) {
+        const bool usable = rate[k] >= 0.0f;
+        const bool is_near = usable && rate[k] < thr;
+        const bool is_far = usable && !is_near;
+        if (has_ref) {
+            // far chunks go to the second block first; the first block takes near ones, or far ones that are left
+            if (is_far && pick_b.size() < n_b) pick_b.push_back(k);
+            else if ((a_is_near ? is_near : is_far) && pick_a.size() < n_a) pick_a.push_back(k);
+            else rest.push_back(k);
+        } else if ((a_is_near ? is_near : is_far) && pick_a.size() < n_a) pick_a.push_back(k);
+        else if ((a_is_near ? is_far : is_near) && pick_b.size() < n_b) pick_b.push_back(k);
+        else rest.push_back(k);
+    }
+    const size_t good_b = pick_b.size();
+    // not enough of a kind: the blocks are completed with whatever else was taken, and with fresh chunks
+    for (int which = 0; which < 2; ++which) {
+        std::vector<size_t>& pick = which ? pick_b : pick_a;
+        const size_t want = which ? n_b : n_a;
+        while (pick.size() < want && !rest.empty()) {
+            pick.push_back(rest.back());
+            rest.pop_back();
+        }
+    }
+    (void)hipStreamSynchronize(stream);
+    // ---- the final blocks: the picked chunks side by side in address ranges of their own
+    void* va[2] = {nullptr, nullptr};
+    std::vector<hipMemGenericAllocationHandle_t> mine[2];
+    const std::vector<size_t>* picks[2] = {&pick_a, &pick_b};
+    const size_t want_n[2] = {n_a, n_b};
+    size_t n_mapped[2] = {0, 0};
+    hipError_t e = hipSuccess;
+    for (size_t k = 0; k < chunks.size() && e == hipSuccess; ++k) e = hipMemUnmap((uint8_t*)scratch + k * C, C);
+    std::vector<bool> taken(chunks.size(), false);
+    for (int which = 0; which < 2 && e == hipSuccess; ++which) {
+        e = hipMemAddressReserve(&va[which], want_n[which] * C, 0, nullptr, 0);
+        if (e != hipSuccess) { va[which] = nullptr; break; }
+        for (size_t k : *picks[which]) {
+            mine[which].push_back(chunks[k]);
+            taken[k] = true;
+        }
+        while (mine[which].size() < want_n[which] && e == hipSuccess) {   // the search ended early: fresh chunks
+            hipMemGenericAllocationHandle_t hnd;
+            e = hipMemCreate(&hnd, C, &prop, 0);
+            if (e == hipSuccess) mine[which].push_back(hnd);
+        }
+        for (size_t i = 0; i < mine[which].size() && e == hipSuccess; ++i) {
+            e = hipMemMap((uint8_t*)va[which] + i * C, C, 0, mine[which][i], 0);
+            if (e == hipSuccess) {
+                ++n_mapped[which];
+                e = hipMemSetAccess((uint8_t*)va[which] + i * C, C, &access, 1);
+            }
+        }
+        if (e == hipSuccess) e = hipMemsetAsync(va[which], 0, want_n[which] * C, stream);
+    }
+    // chunks that serve neither block go back to the driver, and so does the scratch range
+    for (size_t k = 0; k < chunks.size(); ++k)
+        if (!taken[k]) (void)hipMemRelease(chunks[k]);
+    (void)hipMemAddressFree(scratch, n_max * C);
+    if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    if (e != hipSuccess) {
+        (void)hipDeviceSynchronize();
+        for (int which = 0; which < 2; ++which)
+            (void)pair_teardown(va[which], va[which] ? want_n[which] * C : 0, mine[which], n_mapped[which]);
+        (void)hipGetLastError();
+        return fail(e == hipErrorOutOfMemory ? RT_ENOMEM : RT_EHIP, "assembling the two blocks failed: %s",
+                    hipGetErrorString(e));
+    }
+    {
+        std::lock_guard<std::mutex> lock(g_pair_mutex);
+        for (int which = 0; which < 2; ++which) {
+            PairBlock pb;
+            pb.bytes = want_n[which] * C;
+            pb.device = h->device;
+            pb.chunks = std::move(mine[which]);
+            g_pair_blocks[va[which]] = std::move(pb);
+        }
+    }
+    *a_out = va[0];
+    *b_out = va[1];
+    report[0] = complete ? 1.0 : 0.0;
+    report[1] = (double)good_b / (double)n_b;          // share of the second block that lies apart from the first
+    report[2] = (double)rate.size();                    // chunks taken and probed
+    report[3] = elapsed();
+    report[4] = lo;                                     // GB/s of the probe with everything in one region ...
+    report[5] = hi;                                     // ... and with ema_squared in another
+    report[6] = (double)ended;
+    report[7] = a_is_near ? 1.0 : 0.0;
+    return RT_OK;
+}
+
 int rt_dev_release(rt_handle* h, void* p) {
     if (!p) return RT_OK;
+    {
+        std::unique_lock<std::mutex> lock(g_pair_mutex);
+        auto it = g_pair_blocks.find(p);
+        if (it != g_pair_blocks.end()) {
+            PairBlock pb = std::move(it->second);
+            g_pair_blocks.erase(it);
+            lock.unlock();
+            HIP_TRY(hipSetDevice(pb.device));
+            HIP_TRY(hipDeviceSynchronize());   // nothing may still be using the block when its mapping goes
+            const hipError_t e = pair_teardown(p, pb.bytes, pb.chunks, pb.chunks.size());
+            if (e != hipSuccess) return fail(RT_EHIP, "releasing a block of rt_dev_hold_pair: %s", hipGetErrorString(e));
+            return RT_OK;
+        }
+    }
     if (h) HIP_TRY(hipSetDevice(h->device));
     HIP_TRY(hipFree(p));  // the runtime finds the owning device by the address
     return RT_OK;

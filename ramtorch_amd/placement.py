@@ -71,13 +71,73 @@ class _HeldBlock:
             pass  # interpreter shutdown: the process is about to return the memory anyway
 
 
+def reference_arrays(params, device):
+    """(address, address, address, elements) of three disjoint arrays inside the largest contiguous
+    parameter on ``device`` for the chunk-wise placement to probe with (they are written back bit for
+    bit as they are), or None when no parameter is large enough."""
+    best = None
+    for p in params:
+        if p.is_cuda and p.device == device and p.is_contiguous() and p.data_ptr() % 16 == 0:
+            if best is None or p.numel() * p.element_size() > best.numel() * best.element_size():
+                best = p
+    if best is None:
+        return None
+    third = best.numel() * best.element_size() // 3 // 16 * 16    # bytes per array, 16-byte granules
+    elems = min(third // 2, 1 << 27) // 8192 * 8192                # 16-bit elements per array
+    if elems < (1 << 25):
+        return None
+    return best.data_ptr(), best.data_ptr() + third, best.data_ptr() + 2 * third, elems
+
+
+_ENDED = {0: None, 1: "the search reached the memory it may occupy", 2: "the search reached its time limit",
+          3: "the device had no free chunk left"}
+
+
+def _place_pair_by_chunks(handle, device, bytes_a, bytes_b, free0, max_filler_bytes, max_fraction_of_free, max_seconds,
+                          stream, report, log, ref):
+    """The two pools from individually probed 1 GiB chunks (see rt_dev_hold_pair); None when the runtime
+    cannot do that (the caller then searches with whole allocations)."""
+    chunk = GIB
+    need = -(-bytes_a // chunk) * chunk + -(-bytes_b // chunk) * chunk
+    extra = min(max_filler_bytes, int(max_fraction_of_free * max(0, free0 - need)))
+    if need + 2 * GIB > free0:
+        return None
+    try:
+        a_ptr, b_ptr, rep = handle.dev_hold_pair(bytes_a, bytes_b, extra, max_seconds, ref, stream)
+    except N.NativeError as e:
+        if log:
+            log(f"chunk-wise placement not used: {e}")
+        return None
+    a = _HeldBlock(a_ptr, -(-bytes_a // chunk) * chunk, device).tensor()[:bytes_a]
+    b = _HeldBlock(b_ptr, -(-bytes_b // chunk) * chunk, device).tensor()[:bytes_b]
+    report.update(placed=bool(rep[0]), filler_GiB=max(0.0, rep[2] * chunk - need) / GIB, tries=int(rep[2]),
+                  same_GBps=rep[4], cross_GBps=rep[5], by_chunks=True, share_apart=rep[1])
+    reason = _ENDED.get(int(rep[6]))
+    if reason and not rep[0]:
+        report["reason"] = f"{reason}; {100 * rep[1]:.0f} % of the second pool lies apart from the first"
+    res = split_probe(handle, a.data_ptr(), bytes_a, b.data_ptr(), bytes_b, device, stream)
+    if res is not None:   # what the pools themselves show, beginning / middle / end
+        report.update(same_GBps=sum(x[0] for x in res) / len(res), cross_GBps=sum(x[1] for x in res) / len(res))
+    return a, b
+
+
 def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: int, *,
                min_gain: float = 1.05, min_gain_anywhere: float = 1.02, filler_bytes: int = 2 * GIB,
                step_bytes: int = 16 * GIB, max_filler_bytes: int = 112 * GIB, max_fraction_of_free: float = 0.5,
-               max_seconds: float = 1.0, log: Optional[Callable[[str], None]] = None):
+               max_seconds: float = 1.0, by_chunks: bool = True, ref=None,
+               log: Optional[Callable[[str], None]] = None):
     """Two zeroed byte pools on ``device`` such that arrays in the second are, as far as it can be
     arranged, in another HBM region than the corresponding arrays in the first.  Returns
     (pool_a, pool_b, report).
+
+    Pools of at least 1 GiB are first built chunk by chunk (``by_chunks``, ``rt_dev_hold_pair``): physical
+    chunks of 1 GiB are taken one at a time, each is probed against the first one, and the two pools
+    are mapped from chunks of the two kinds -- which also works in a process whose earlier
+    allocations left the free memory in scattered order, where a single allocation of many GiB
+    straddles regions.  Both pools are then memory held through the library.  ``ref``: three disjoint
+    arrays in the memory of the parameters (see ``reference_arrays``):
+    the first pool then lies where the parameters are and the second elsewhere.  What follows describes
+    the search that is used when that is not available or does not apply.
 
     The place right behind the first pool is tried first.  A place is taken when the probe shows
     the gain there: ``min_gain`` on the mean over the beginning, the middle and the end of the pools,
@@ -105,6 +165,12 @@ def place_pair(handle: N.Handle, device: torch.device, bytes_a: int, bytes_b: in
     report = {"placed": False, "filler_GiB": 0.0, "same_GBps": None, "cross_GBps": None, "tries": 0, "seconds": 0.0,
               "reason": None}
     free0, _ = torch.cuda.mem_get_info(device)
+    if by_chunks and min(bytes_a, bytes_b) >= GIB:
+        got = _place_pair_by_chunks(handle, device, bytes_a, bytes_b, free0, max_filler_bytes, max_fraction_of_free,
+                                    max_seconds, stream, report, log, ref)
+        if got is not None:
+            report["seconds"] = time.monotonic() - t0
+            return got[0], got[1], report
     a = zeros(bytes_a)
     # Pools under 1 GiB are not worth occupying -- and having the driver clear afterwards -- a hundred
     # GiB for: their launches are short and the probe on them says little.  From 1 GiB on the place

@@ -358,7 +358,8 @@ class AdamW(Optimizer):
         N.lib()
         with torch.cuda.device(dev):
             pool_m, pool_v, report = placement.place_pair(_handle(dev.index), dev, total * esize["ema"],
-                                                          total * esize["ema_squared"])
+                                                          total * esize["ema_squared"],
+                                                          ref=placement.reference_arrays(params, dev))
         self.state_placement_report = report
         self._state_pools = {"ema": pool_m, "ema_squared": pool_v, "slots": slots}
         for k, p in enumerate(params):
