@@ -129,13 +129,16 @@ class AdamW(Optimizer):
             ``state_pool_min_bytes`` per kind, "auto" carves all ``ema`` tensors out of one
             pool and all ``ema_squared`` tensors out of another and places the two pools in
             different HBM regions, found by measurement at construction (see
-            ``ramtorch_amd/placement.py``; the outcome is in ``state_placement_report``).
-            While it searches, the constructor occupies up to half of the free device memory
-            (at most 112 GiB, for pools under 1 GiB eight times their size; for about a second) through the library and gives all of it back
-            (the driver clears released memory in the background at about 33 GB/s, and until it
-            is done device-wide memory traffic runs about 1 % slower: the first seconds of a run);
-            torch's caching allocator only ever sees the first pool (the second is memory held
-            through the library, wrapped as a tensor, and released with its last view).
+            ``ramtorch_amd/placement.py``; the outcome is in ``state_placement_report``): free device
+            memory is taken in chunks of 1 GiB through the library (up to half of what is free, at most
+            112 GiB beyond the pools, for up to a second), every chunk is probed with the update's
+            traffic against the largest parameter's own memory, the pools are mapped from chunks of
+            the two kinds and the rest is given back.  The probe writes the parameter back bit for bit
+            as it is; nothing else should be writing parameters meanwhile.
+            (The driver clears released memory in the background at about 33 GB/s, and until it
+            is done device-wide memory traffic runs about 1 % slower: the first seconds of a run.)
+            torch's caching allocator never sees the pools (memory held through the library,
+            wrapped as tensors, released with their last views).
             "plain" allocates every state tensor on its own, as the reference does.
     """
 

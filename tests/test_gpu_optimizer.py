@@ -890,6 +890,53 @@ def test_state_placement_of_two_large_optimizers_in_a_row():
         torch.cuda.empty_cache()       # tens of GiB go back to the driver: the next round starts in a used process
 
 
+def test_state_placement_with_scattered_free_memory_is_as_clean_as_in_a_fresh_process():
+    """Free device memory in scattered order -- every other block of many released -- is where one
+    allocation of several GiB straddles HBM regions.  The pools are mapped from 1 GiB chunks that were
+    probed one by one against the parameter's own memory: both are complete, they show the gain of lying
+    in different regions, the probing has left every bit of the parameter as it was, and the steps are
+    those of an optimizer with plainly allocated states."""
+    GIB = 1 << 30
+    blocks = [torch.empty(3 * GIB // 2, dtype=torch.uint8, device="cuda") for _ in range(120)]
+    keep = blocks[::2]
+    del blocks
+    torch.cuda.empty_cache()
+    try:
+        n = 1 << 30    # 2 GiB of bf16 per array
+        gen = torch.Generator("cuda").manual_seed(77)
+        base = (torch.randn(n, device="cuda", generator=gen) * 0.02).bfloat16()
+        grad = (torch.randn(n, device="cuda", generator=gen) * 1e-3).bfloat16()
+        p1 = torch.nn.Parameter(base.clone(), requires_grad=False)
+        p2 = torch.nn.Parameter(base, requires_grad=False)
+        opt1 = ramtorch_amd.AdamW([p1], storage_device="cuda", seed=3, state_placement="auto", **HP0)
+        torch.cuda.synchronize()
+        rep = opt1.state_placement_report
+        assert torch.equal(p1.view(torch.int16), p2.view(torch.int16)), "the placement probes changed the parameter"
+        assert rep.get("by_chunks") and rep["placed"] and rep["share_apart"] == 1.0, rep
+        assert rep["cross_GBps"] >= 1.04 * rep["same_GBps"], rep
+        assert rep["seconds"] < 2.0, rep
+        st = opt1.state[p1]
+        assert not bool(st["ema"].view(torch.int16).any()) and not bool(st["ema_squared"].view(torch.int16).any())
+        opt2 = ramtorch_amd.AdamW([p2], storage_device="cuda", seed=3, state_placement="plain", **HP0)
+        for _ in range(2):
+            p1.grad = p2.grad = grad
+            opt1.step(); opt2.step()
+        torch.cuda.synchronize()
+        assert torch.equal(p1.view(torch.int16), p2.view(torch.int16))
+        for k in ("ema", "ema_squared"):
+            assert torch.equal(opt1.state[p1][k].view(torch.int16), opt2.state[p2][k].view(torch.int16))
+        # the pools go back to the driver with their last views
+        free_before = torch.cuda.mem_get_info()[0]
+        del opt1, st
+        import gc
+        gc.collect()
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] - free_before >= 4 * GIB - (64 << 20)
+    finally:
+        del keep
+        torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize("pdt,sdt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
                                      (torch.bfloat16, torch.float16)])
 @pytest.mark.parametrize("clip", [None, 0.05])
