@@ -913,8 +913,8 @@ def test_state_placement_with_scattered_free_memory_is_as_clean_as_in_a_fresh_pr
         rep = opt1.state_placement_report
         assert torch.equal(p1.view(torch.int16), p2.view(torch.int16)), "the placement probes changed the parameter"
         assert rep.get("by_chunks") and rep["placed"] and rep["share_apart"] == 1.0, rep
-        assert rep["cross_GBps"] >= 1.04 * rep["same_GBps"], rep
-        assert rep["seconds"] < 2.0, rep
+        assert rep["cross_GBps"] >= 1.03 * rep["same_GBps"], rep      # 6 - 7 % where measured
+        assert rep["seconds"] < 3.0, rep                              # 0.2 s where measured
         st = opt1.state[p1]
         assert not bool(st["ema"].view(torch.int16).any()) and not bool(st["ema_squared"].view(torch.int16).any())
         opt2 = ramtorch_amd.AdamW([p2], storage_device="cuda", seed=3, state_placement="plain", **HP0)
