@@ -71,10 +71,19 @@ class _HeldBlock:
             pass  # interpreter shutdown: the process is about to return the memory anyway
 
 
+#: Whether the optimizer lets the chunk-wise placement probe with the parameters' own memory (it writes
+#: them back bit for bit as they are).  Set to False when something else may be writing parameters while
+#: optimizers are constructed: chunks are then sorted relative to the first chunk taken, which keeps the
+#: two pools apart from each other but not necessarily the first one with the parameters.
+PROBE_WITH_PARAMETERS = True
+
+
 def reference_arrays(params, device):
     """(address, address, address, elements) of three disjoint arrays inside the largest contiguous
     parameter on ``device`` for the chunk-wise placement to probe with (they are written back bit for
     bit as they are), or None when no parameter is large enough."""
+    if not PROBE_WITH_PARAMETERS:
+        return None
     best = None
     for p in params:
         if p.is_cuda and p.device == device and p.is_contiguous() and p.data_ptr() % 16 == 0:
