@@ -937,6 +937,30 @@ def test_state_placement_with_scattered_free_memory_is_as_clean_as_in_a_fresh_pr
         torch.cuda.empty_cache()
 
 
+def test_state_placement_without_probing_parameter_memory(monkeypatch):
+    """placement.PROBE_WITH_PARAMETERS = False: chunks are sorted relative to the first chunk taken; the pools
+    still come from individually probed chunks, lie apart from each other, hold zeros, and step like plain states."""
+    from ramtorch_amd import placement
+    monkeypatch.setattr(placement, "PROBE_WITH_PARAMETERS", False)
+    n = 1 << 30
+    gen = torch.Generator("cuda").manual_seed(78)
+    base = (torch.randn(n, device="cuda", generator=gen) * 0.02).bfloat16()
+    grad = (torch.randn(n, device="cuda", generator=gen) * 1e-3).bfloat16()
+    p1 = torch.nn.Parameter(base.clone(), requires_grad=False)
+    p2 = torch.nn.Parameter(base, requires_grad=False)
+    opt1 = ramtorch_amd.AdamW([p1], storage_device="cuda", seed=3, state_placement="auto", **HP0)
+    rep = opt1.state_placement_report
+    assert rep.get("by_chunks") and (rep["placed"] or rep["reason"]), rep
+    if rep["placed"]:
+        assert rep["cross_GBps"] >= 1.03 * rep["same_GBps"], rep
+    opt2 = ramtorch_amd.AdamW([p2], storage_device="cuda", seed=3, state_placement="plain", **HP0)
+    p1.grad = p2.grad = grad
+    opt1.step(); opt2.step()
+    torch.cuda.synchronize()
+    assert torch.equal(p1.view(torch.int16), p2.view(torch.int16))
+    assert torch.equal(opt1.state[p1]["ema_squared"].view(torch.int16), opt2.state[p2]["ema_squared"].view(torch.int16))
+
+
 @pytest.mark.parametrize("pdt,sdt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
                                      (torch.bfloat16, torch.float16)])
 @pytest.mark.parametrize("clip", [None, 0.05])
