@@ -2101,6 +2101,7 @@ int rt_dev_hold_pair(rt_handle* h, uint64_t bytes_a, uint64_t bytes_b, uint64_t 
         if (has_ref) return far_n >= n_b && near_n >= n_a;
         return (near_n >= n_a && far_n >= n_b) || (far_n >= n_a && near_n >= n_b);
     };
+    double create_seconds = 0.0;   // spent inside hipMemCreate so far
     int ended = 0;   // 0: both blocks complete, 1: memory limit, 2: time limit, 3: no more free chunks
     bool complete = false;
     while (true) {
@@ -2110,9 +2111,16 @@ int rt_dev_hold_pair(rt_handle* h, uint64_t bytes_a, uint64_t bytes_b, uint64_t 
             break;
         }
         if (chunks.size() >= n_max) { ended = 1; break; }
-        if (!chunks.empty() && elapsed() > max_seconds) { ended = 2; break; }
+        // Time: what has passed, plus what giving the surplus chunks back will take.  While the driver is still
+        // clearing memory that was freed shortly before, taking a chunk and giving one back cost about 30 ms each
+        // (next to nothing otherwise); the cost of taking them is the estimate for giving them back.
+        const size_t surplus = chunks.size() > n_a + n_b ? chunks.size() - (n_a + n_b) : 0;
+        const double per_chunk = chunks.empty() ? 0.0 : create_seconds / (double)chunks.size();
+        if (!chunks.empty() && elapsed() + (double)surplus * per_chunk > max_seconds) { ended = 2; break; }
         hipMemGenericAllocationHandle_t hnd;
+        const double t_create = elapsed();
         hipError_t e = hipMemCreate(&hnd, C, &prop, 0);
+        create_seconds += elapsed() - t_create;
         if (e != hipSuccess) {
             (void)hipGetLastError();
             ended = 3;
