@@ -374,7 +374,10 @@ int rt_dev_release(rt_handle* h, void* p);
  * of its own.  Chunk by chunk, so it works as well in a process whose earlier
  * allocations have left the free memory in scattered order, where one large
  * allocation straddles regions.  On the way the search holds at most
- * max_extra_bytes more than the two blocks and gives up after max_seconds;
+ * max_extra_bytes more than the two blocks and gives up when taking and
+ * probing chunks beyond those of the blocks has cost max_seconds (two and a
+ * half times that while the driver hands out chunks slowly because it is
+ * still clearing memory that was given back shortly before);
  * blocks it could not complete from the right kind of chunk are completed with
  * others.  Each block is given back with rt_dev_release (which waits for the
  * device first).  RT_EUNSUPPORTED when the runtime has no such allocations.
@@ -389,13 +392,16 @@ int rt_dev_release(rt_handle* h, void* p);
  * second as well), *b from the second, and an update never has p, ema and
  * ema_squared in one region nor, with *a complete, in three.  The probe
  * writes the reference arrays back bit for bit as they are (it stores p ^ g
- * with g zero); nothing else may write them while the call runs.
+ * with g zero); nothing else may write them while the call runs.  Reference
+ * arrays that do not lie in one region themselves (the probe with all of
+ * them runs faster than with all arrays inside one chunk) are not used.
  *   report[0] = 1 when both blocks are wholly of their kind, else 0
  *   report[1] = share of the second block that lies apart from the first
  *   report[2] = chunks taken and probed       report[3] = seconds
  *   report[4], report[5] = GB/s of the probe within one region / across two
  *   report[6] = why the search ended: 0 complete, 1 memory limit, 2 time limit, 3 no free chunk left
- *   report[7] = 1 when *a is the block in the first chunk's region
+ *   report[7] = 2 when the kinds were told apart relative to the reference arrays (*a lies with them), else
+ *               1 when *a is the block in the first chunk's region, 0 when *b is
  */
 int rt_dev_hold_pair(rt_handle* h, uint64_t bytes_a, uint64_t bytes_b, uint64_t max_extra_bytes, double max_seconds,
                      void* ref_p, void* ref_m, void* ref_v, uint64_t ref_elems, void** a, void** b,

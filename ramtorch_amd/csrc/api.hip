@@ -2036,17 +2036,13 @@ int rt_dev_hold_pair(rt_handle* h, uint64_t bytes_a, uint64_t bytes_b, uint64_t 
     // stand in the first chunk.  With them, p and ema are the caller's own arrays -- parameter memory, so
     // that "the first kind" means "where the parameters are"; the probe writes p ^ g and ema ^ g back and
     // g is a zeroed part of the first chunk, so every bit of them stays as it is.
-    auto probe = [&](void* v, float* gbps) -> hipError_t {
-        uint8_t* base = (uint8_t*)scratch;
-        const size_t arr = probe_elems * 2;
-        const uint64_t pp = has_ref ? (uint64_t)ref_p : (uint64_t)base;
-        const uint64_t gg = has_ref ? (uint64_t)base : (uint64_t)(base + arr);
-        const uint64_t mm = has_ref ? (uint64_t)ref_m : (uint64_t)(base + 2 * arr);
+    bool use_ref = has_ref;   // dropped when the reference arrays turn out not to lie in one region themselves
+    auto probe4 = [&](uint64_t pp, uint64_t gg, uint64_t mm, uint64_t vv, float* gbps) -> hipError_t {
         const dim3 grid((uint32_t)(probe_elems / kChunkElems));
-        hipLaunchKernelGGL(stream_probe_kernel, grid, dim3(kThreads), 0, stream, pp, gg, mm, (uint64_t)v);
+        hipLaunchKernelGGL(stream_probe_kernel, grid, dim3(kThreads), 0, stream, pp, gg, mm, vv);
         hipError_t e = hipEventRecord(h->t0, stream);
         for (int r = 0; r < 3 && e == hipSuccess; ++r)
-            hipLaunchKernelGGL(stream_probe_kernel, grid, dim3(kThreads), 0, stream, pp, gg, mm, (uint64_t)v);
+            hipLaunchKernelGGL(stream_probe_kernel, grid, dim3(kThreads), 0, stream, pp, gg, mm, vv);
         if (e == hipSuccess) e = hipGetLastError();
         if (e == hipSuccess) e = hipEventRecord(h->t1, stream);
         if (e == hipSuccess) e = hipEventSynchronize(h->t1);
@@ -2055,12 +2051,21 @@ int rt_dev_hold_pair(rt_handle* h, uint64_t bytes_a, uint64_t bytes_b, uint64_t 
         if (e == hipSuccess) *gbps = (float)(14.0 * (double)probe_elems * 3 / (ms * 1e-3) / 1e9);
         return e;
     };
+    auto probe = [&](void* v, float* gbps) -> hipError_t {
+        uint8_t* base = (uint8_t*)scratch;
+        const size_t arr = probe_elems * 2;
+        if (use_ref) return probe4((uint64_t)ref_p, (uint64_t)base, (uint64_t)ref_m, (uint64_t)v, gbps);
+        return probe4((uint64_t)base, (uint64_t)(base + arr), (uint64_t)(base + 2 * arr), (uint64_t)v, gbps);
+    };
 
     float lo = 0.0f, hi = 0.0f;   // mean rates of the two kinds of chunk
     size_t near_n = 0, far_n = 0;
     // Two kinds of chunk: those that run at the rate of the first chunk's own region and those that run at the
     // higher rate of another region.  Two-means over the rates seen so far; the kinds count as told apart only
     // when their means differ by 4 % (single probes scatter by 2 - 3 %, the regions differ by 7 %).
+    // (With reference arrays the rates come in three levels, e.g. 5.9 / 6.2 / 6.44 TB/s: the chunk in the
+    // parameters' region; elsewhere, with the gradient's stand-in -- the first chunk -- in a third region; and
+    // elsewhere with it in one of the two.  The lowest level is the first kind, the two others are the second.)
     float ref_level = 0.0f;   // with reference arrays: the rate with ema_squared in parameter memory as well
     auto classify = [&]() -> float {
         near_n = far_n = 0;
@@ -2086,7 +2091,7 @@ int rt_dev_hold_pair(rt_handle* h, uint64_t bytes_a, uint64_t bytes_b, uint64_t 
         // when it runs 3.5 % faster than the probe that has all its arrays inside the parameters' memory.
         float thr = 1e30f;
         if (c2 >= 1.04f * c1) thr = 0.5f * (c1 + c2);
-        else if (has_ref && 0.5f * (c1 + c2) >= 1.035f * ref_level) thr = 0.0f;
+        else if (use_ref && 0.5f * (c1 + c2) >= 1.035f * ref_level) thr = 0.0f;
         for (float r : rate) {
             if (r < 0.0f) continue;
             (r < thr ? near_n : far_n) += 1;
@@ -2098,10 +2103,11 @@ int rt_dev_hold_pair(rt_handle* h, uint64_t bytes_a, uint64_t bytes_b, uint64_t 
     // chunks for that, the search runs to its limits and the first block is completed with chunks from elsewhere
     // (the parameters then have their region to themselves, which is still better than sharing it with both).
     auto is_complete = [&] {
-        if (has_ref) return far_n >= n_b && near_n >= n_a;
+        if (use_ref) return far_n >= n_b && near_n >= n_a;
         return (near_n >= n_a && far_n >= n_b) || (far_n >= n_a && near_n >= n_b);
     };
     double create_seconds = 0.0;   // spent inside hipMemCreate so far
+    double base_seconds = 0.0;     // when the chunks that the blocks need anyway had been taken
     int ended = 0;   // 0: both blocks complete, 1: memory limit, 2: time limit, 3: no more free chunks
     bool complete = false;
     while (true) {
@@ -2111,12 +2117,15 @@ int rt_dev_hold_pair(rt_handle* h, uint64_t bytes_a, uint64_t bytes_b, uint64_t 
             break;
         }
         if (chunks.size() >= n_max) { ended = 1; break; }
-        // Time: what has passed, plus what giving the surplus chunks back will take.  While the driver is still
-        // clearing memory that was freed shortly before, taking a chunk and giving one back cost about 30 ms each
-        // (next to nothing otherwise); the cost of taking them is the estimate for giving them back.
+        // Time.  The chunks that the two blocks consist of have to be taken whatever their kind: the limit is for
+        // what the search costs beyond that.  While the driver is still clearing memory that was given back shortly
+        // before (by this process or by one that has just ended), it hands out chunks only as fast as it clears
+        // them, about 30 ms per GiB instead of next to nothing, and takes as long to take them back; the search is
+        // then given two and a half times as long, because a place found once serves every step that follows.
         const size_t surplus = chunks.size() > n_a + n_b ? chunks.size() - (n_a + n_b) : 0;
         const double per_chunk = chunks.empty() ? 0.0 : create_seconds / (double)chunks.size();
-        if (!chunks.empty() && elapsed() + (double)surplus * per_chunk > max_seconds) { ended = 2; break; }
+        if (chunks.size() == n_a + n_b) base_seconds = elapsed();
+        if (surplus && elapsed() - base_seconds > (per_chunk > 0.012 ? 2.5 : 1.0) * max_seconds) { ended = 2; break; }
         hipMemGenericAllocationHandle_t hnd;
         const double t_create = elapsed();
         hipError_t e = hipMemCreate(&hnd, C, &prop, 0);
@@ -2137,14 +2146,27 @@ int rt_dev_hold_pair(rt_handle* h, uint64_t bytes_a, uint64_t bytes_b, uint64_t 
         if (e != hipSuccess) return fail_all(RT_EHIP, "hipMemSetAccess", e);
         float r0 = 0.0f, r1 = 0.0f;
         const size_t arr = probe_elems * 2;
-        if (chunks.size() == 1 && has_ref) {
-            // the first chunk holds the zeroed stand-in for the gradient at its beginning
+        if (chunks.size() == 1 && use_ref) {
+            // The first chunk holds the zeroed stand-in for the gradient at its beginning.  First of all the
+            // reference arrays are checked against the chunk: with all four arrays inside one chunk the probe runs
+            // at the rate of a single region, and with all of them inside the parameters' memory it must run no
+            // faster -- if it does, that memory lies across a region boundary itself and is no reference.
             e = hipMemsetAsync(at, 0, arr, stream);
-            float l0 = 0.0f, l1 = 0.0f;
+            float l0 = 0.0f, l1 = 0.0f, own = 0.0f;
             if (e == hipSuccess) e = probe(ref_v, &l0);
             if (e == hipSuccess) e = probe(ref_v, &l1);
             ref_level = std::max(l0, l1);
-            if (e == hipSuccess) e = probe(at + arr, &r0);
+            for (int rep = 0; rep < 2 && e == hipSuccess; ++rep) {
+                float r = 0.0f;
+                e = probe4((uint64_t)(at + arr), (uint64_t)at, (uint64_t)(at + 2 * arr), (uint64_t)(at + 3 * arr), &r);
+                own = std::max(own, r);
+            }
+            // (two regions differ by 7 %, single probes scatter by 2 - 3 %)
+            if (e == hipSuccess && ref_level > 1.05f * own) use_ref = false;
+        }
+        if (e != hipSuccess) return fail_all(RT_EHIP, "probing a chunk", e);
+        if (chunks.size() == 1 && use_ref) {
+            e = probe(at + arr, &r0);
             if (e == hipSuccess) e = probe(at + C - arr, &r1);
         } else if (chunks.size() == 1) {
             // all four arrays inside the first chunk: the rate of one region
@@ -2163,13 +2185,13 @@ int rt_dev_hold_pair(rt_handle* h, uint64_t bytes_a, uint64_t bytes_b, uint64_t 
     complete = is_complete();
     // Without reference arrays: the block that must lie in one region takes the chunks of the first chunk's kind
     // ("near"), the other takes chunks that are anywhere else -- whichever way round the counts allow.
-    const bool a_is_near = has_ref ? true : !(complete && !(near_n >= n_a && far_n >= n_b));
+    const bool a_is_near = use_ref ? true : !(complete && !(near_n >= n_a && far_n >= n_b));
     std::vector<size_t> pick_a, pick_b, rest;
     for (size_t k = 0; k < chunks.size(); ++k) {
         const bool usable = rate[k] >= 0.0f;
         const bool is_near = usable && rate[k] < thr;
         const bool is_far = usable && !is_near;
-        if (has_ref) {
+        if (use_ref) {
             // far chunks go to the second block first; the first block takes near ones, or far ones that are left
             if (is_far && pick_b.size() < n_b) pick_b.push_back(k);
             else if ((a_is_near ? is_near : is_far) && pick_a.size() < n_a) pick_a.push_back(k);
@@ -2251,7 +2273,7 @@ int rt_dev_hold_pair(rt_handle* h, uint64_t bytes_a, uint64_t bytes_b, uint64_t 
     report[4] = lo;                                     // GB/s of the probe with everything in one region ...
     report[5] = hi;                                     // ... and with ema_squared in another
     report[6] = (double)ended;
-    report[7] = a_is_near ? 1.0 : 0.0;
+    report[7] = use_ref ? 2.0 : a_is_near ? 1.0 : 0.0;
     return RT_OK;
 }
 

@@ -120,7 +120,8 @@ def _place_pair_by_chunks(handle, device, bytes_a, bytes_b, free0, max_filler_by
     a = _HeldBlock(a_ptr, -(-bytes_a // chunk) * chunk, device).tensor()[:bytes_a]
     b = _HeldBlock(b_ptr, -(-bytes_b // chunk) * chunk, device).tensor()[:bytes_b]
     report.update(placed=bool(rep[0]), filler_GiB=max(0.0, rep[2] * chunk - need) / GIB, tries=int(rep[2]),
-                  same_GBps=rep[4], cross_GBps=rep[5], by_chunks=True, share_apart=rep[1])
+                  same_GBps=rep[4], cross_GBps=rep[5], by_chunks=True, share_apart=rep[1],
+                  relative_to_parameters=rep[7] == 2.0)
     reason = _ENDED.get(int(rep[6]))
     if reason and not rep[0]:
         report["reason"] = f"{reason}; {100 * rep[1]:.0f} % of the second pool lies apart from the first"
